@@ -1,0 +1,148 @@
+/*
+ * mtj_abi.h - C ABI of the MI355X (gfx950) GPT-J forward/decode kernels.
+ *
+ * The reference (kingoflolz/mesh-transformer-jax) is pure Python on JAX: it has no FFI of its own,
+ * so these entry points are what a binding for its generate path would bind.  Each one cites the
+ * reference code whose XLA-generated kernels it replaces (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing here allocates, frees or
+ *     keeps a pointer after returning;
+ *   - every call is asynchronous on `stream` (a hipStream_t passed as void*), never synchronises,
+ *     and is safe to record into a HIP graph: per-step scalars (positions) are read from device memory;
+ *   - return value: 0 on success, a negative MTJ_E* code otherwise; mtj_last_error() returns the
+ *     message of the calling thread's last failure;
+ *   - activations are float32 unless `dtype` says otherwise; `dtype` selects the storage type of
+ *     weights / K,V cache / GEMM inputs: MTJ_F32 (exact path) or MTJ_BF16;
+ *   - "packed" weights are row-major [N_out, K_in] (K contiguous), i.e. the transpose of haiku's
+ *     [in, out]; mtj_pack_weight builds them, with row/column offsets so that q|v|k|fc_in are
+ *     concatenated along N and out|fc_out along K.
+ */
+#ifndef MTJ_ABI_H
+#define MTJ_ABI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MTJ_ABI_VERSION 1
+
+enum { MTJ_F32 = 0, MTJ_BF16 = 1 };
+
+enum {
+  MTJ_OK = 0,
+  MTJ_EINVAL = -1,   /* bad shape / argument (mirrors the reference's Python asserts) */
+  MTJ_EALIGN = -2,   /* pointer or leading dimension not 16-byte aligned */
+  MTJ_EDTYPE = -3,   /* unsupported dtype */
+  MTJ_EHIP = -4,     /* HIP launch error, message holds hipGetErrorString */
+  MTJ_ELIMIT = -5    /* size beyond what the kernel supports (e.g. LDS capacity) */
+};
+
+int mtj_version(void);
+const char* mtj_last_error(void);
+
+/* Epilogues of mtj_gemm / mtj_gemv. */
+enum {
+  MTJ_EPI_STORE = 0,  /* out[m, n] = acc (+ bias[n])                           (ProjectionShard linear, layers.py:559-563) */
+  MTJ_EPI_RESID = 1,  /* x[m, n] += acc + bias[n], float32 in place            (layers.py:313 + transformer_shard.py:92,112) */
+  MTJ_EPI_INPROJ = 2  /* fused q|v|k|fc_in: RoPE(q), RoPE(k) -> cache, v -> cache, gelu(fc_in + b1)
+                         (layers.py:292-297, 261-273, 287-289, 325-326) */
+};
+
+/*
+ * Geometry and destinations of the fused input projection.  Row m of the GEMM is token t = m % Tp of
+ * sequence b = m / Tp, at absolute position pos = pos0[b] + t; rows with pos < 0 are left padding and
+ * write nothing to the cache.  Output columns: [0,d) q, [d,2d) v, [2d,3d) k, [3d,3d+F) fc_in.
+ */
+typedef struct {
+  int32_t n_heads, d_head, rotary_dims; /* H, dh, r (r even, r <= dh)                                   */
+  int32_t Tp;                           /* tokens per sequence in this call (1 at decode)              */
+  int32_t Tcap;                         /* K/V window capacity in slots; slot = pos % Tcap             */
+  int32_t max_pos;                      /* rows of the sin/cos tables                                  */
+  const int32_t* pos0;                  /* [B] position of the first row of each sequence              */
+  const float* sin_tab;                 /* [max_pos, r/2] float32, rounded once from float64           */
+  const float* cos_tab;                 /* [max_pos, r/2]                                              */
+  void* q;                              /* [B, H, Tp, dh] in q_dtype                                   */
+  int32_t q_dtype;                      /* MTJ_F32 (decode attention reads float32 q) or MTJ_BF16      */
+  void* k_cache;                        /* [B, H, Tcap, dh] dtype, rotated keys                        */
+  void* v_cache;                        /* [B, H, Tcap, dh] dtype                                      */
+  void* v_t;                            /* optional [B, H, dh, ldvt] dtype: V transposed, for prefill  */
+  int64_t ldvt;                         /* row length of v_t (>= Tp, multiple of 8)                    */
+  void* act;                            /* [M, ld_act]: gelu(fc_in) goes to columns [d, d+F)           */
+  int64_t ld_act;
+  int32_t act_dtype;                    /* MTJ_F32 or MTJ_BF16                                         */
+} mtj_inproj;
+
+/*
+ * Transpose-pack a haiku [K, N] weight (row stride src_ld) into dst[(n_off + n) * K_total + k_off + k].
+ * Replaces nothing in the reference; it is the layout change that lets q|v|k|fc_in (layers.py:249-256)
+ * run as one GEMM and out|fc_out (layers.py:253-258) as another.
+ */
+int mtj_pack_weight(const void* src, int64_t src_ld, int64_t K, int64_t N, void* dst, int64_t K_total,
+                    int64_t n_off, int64_t k_off, int dtype, void* stream);
+
+/* out[m, :] = W[tok[m], :] + b  (EmbeddingShard.__call__, layers.py:187-202: one_hot @ W + b).
+ * W is the tree leaf itself, [V, d] in `dtype`; b float32 [d]; out float32 [M, d].
+ * Token ids >= n_vocab give a zero row plus bias, as an all-zero one-hot row would. */
+int mtj_embed(const int32_t* tok, int64_t M, const void* W, const float* b, int64_t n_vocab, int64_t d,
+              int dtype, float* out, void* stream);
+
+/* ReplicatedLayerNorm.__call__, layers.py:17-36 (biased variance, eps 1e-5 inside rsqrt).
+ * x float32 [M, d] (row stride d); out [M, d] in out_dtype. */
+int mtj_layernorm(const float* x, const float* scale, const float* offset, int64_t M, int64_t d,
+                  void* out, int out_dtype, void* stream);
+
+/* C = A[M, K] (dtype, row stride lda) x W[N, K]^T (packed, dtype) with epilogue `epi`.
+ * hk.Linear call sites: layers.py:249-258, 559.  MFMA kernel; bias is float32 [N] or NULL.
+ * STORE: out [M, ldo] in out_dtype.  RESID: out float32 [M, ldo].  INPROJ: `ip` non-NULL, bias = b1 [F]. */
+int mtj_gemm(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
+             int dtype, int epi, void* out, int64_t ldo, int out_dtype, const mtj_inproj* ip, void* stream);
+
+/* Batch-1 decode matrix-vector product: y = f(x) @ W^T with float32 activations and float32 accumulation
+ * (jnp.dot(f32, bf16) semantics of hk.Linear at decode, layers.py:316-344).  x float32 [K].
+ * If ln_scale != NULL the kernel first applies LayerNorm(x) (layers.py:17-36) - x then has K = d entries.
+ * Same epilogues as mtj_gemm with M = 1. */
+int mtj_gemv(const float* x, const float* ln_scale, const float* ln_offset, const void* W, const float* bias,
+             int64_t N, int64_t K, int dtype, int epi, void* out, int out_dtype, const mtj_inproj* ip,
+             void* stream);
+
+/* Causal self-attention over a left-padded rectangle (self_attn + masks of get_init_decode_state,
+ * layers.py:260-285, 347-366).  q [B,H,Tp,dh], k_cache [B,H,Tcap,dh] (rotated), v_t [B,H,dh,ldvt];
+ * out[m, h*dh + c] with row stride ld_out, dtype.  Scores are divided by sqrt(dh) after the dot;
+ * masked keys contribute exactly 0 (exp(-1e10 - max) underflows in float32).  Padding rows get zeros. */
+int mtj_attn_prefill(const void* q, const void* k_cache, const void* v_t, const int32_t* pos0, int64_t B,
+                     int64_t H, int64_t Tp, int64_t Tcap, int64_t dh, int64_t ldvt, void* out, int64_t ld_out,
+                     int dtype, void* stream);
+
+/* One-token attention over the K/V window (decode_once, layers.py:316-344): for sequence b the valid
+ * slots are [0, min(pos[b]+1, Tcap)).  q float32 [B,H,dh]; caches in `dtype`; out [B, ld_out] in out_dtype
+ * (columns h*dh + c).  `work` needs mtj_attn_decode_work_bytes(B, H, dh, Tcap) bytes. */
+int64_t mtj_attn_decode_work_bytes(int64_t B, int64_t H, int64_t dh, int64_t Tcap);
+int mtj_attn_decode(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,
+                    int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
+                    void* work, void* stream);
+
+/* Greedy sampler through the reference's sampler contract (transformer_shard.py:203): lowest index among
+ * maxima.  Writes tok[b], out_tokens[b * ld_tokens + (pos[b] - pos_start[b])], then pos[b] += 1. */
+int mtj_sample_greedy(const float* logits, int64_t B, int64_t V, int32_t* tok, int32_t* out_tokens,
+                      int64_t ld_tokens, int32_t* pos, const int32_t* pos_start, void* stream);
+
+/* nucleaus_sample (sampling.py:10-44) with the Gumbel draw replaced by an inverse-CDF draw from
+ * host-supplied uniforms: filter on the RAW logits (optional top_k, then top_p, float64 softmax and
+ * running sum over the stable descending order, ties: higher id first), then weights
+ * exp(filtered/temp - max) in float64 and the first token whose running weight exceeds u * total.
+ * top_p, temp: float64 [B]; top_k: int32 [B] or NULL; uniforms: float64 [B, ld_u], column = step index.
+ * keep_mask (optional) uint8 [B, V]: 1 where the filter left the logit untouched.
+ * filtered (optional) float32 [B, V]: the filter's output.  `work` needs mtj_sample_work_bytes(B, V). */
+int64_t mtj_sample_work_bytes(int64_t B, int64_t V);
+int mtj_sample_nucleus(const float* logits, int64_t B, int64_t V, const double* top_p, const double* temp,
+                       const int32_t* top_k, const double* uniforms, int64_t ld_u, int32_t* tok,
+                       int32_t* out_tokens, int64_t ld_tokens, int32_t* pos, const int32_t* pos_start,
+                       uint8_t* keep_mask, float* filtered, void* work, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MTJ_ABI_H */

@@ -1,0 +1,391 @@
+// Attention: MFMA flash-style prefill over a left-padded rectangle, and one-token decode over the K/V window.
+#include "mtj_common.h"
+
+namespace {
+
+template <typename T> struct mma;
+template <> struct mma<bf16_t> {
+  static constexpr int EPC = 8;
+  typedef uint16_t raw_t;
+  struct frag { bf16x8 v; };
+  __device__ static __forceinline__ frag load(const bf16_t* p) {
+    frag f;
+    f.v = *reinterpret_cast<const bf16x8*>(p);
+    return f;
+  }
+  __device__ static __forceinline__ frag from_floats(const float* p) {  // 8 probabilities -> operand
+    frag f;
+    uint32x4 u;
+    u.x = pack_bf16x2(p[0], p[1]);
+    u.y = pack_bf16x2(p[2], p[3]);
+    u.z = pack_bf16x2(p[4], p[5]);
+    u.w = pack_bf16x2(p[6], p[7]);
+    f.v = *reinterpret_cast<bf16x8*>(&u);
+    return f;
+  }
+  __device__ static __forceinline__ void run(floatx16& c, const frag& a, const frag& b) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
+  }
+};
+template <> struct mma<float> {
+  static constexpr int EPC = 4;
+  typedef uint32_t raw_t;
+  struct frag { float v[8]; };
+  __device__ static __forceinline__ frag load(const float* p) {
+    frag f;
+    const floatx4 lo = *reinterpret_cast<const floatx4*>(p), hi = *reinterpret_cast<const floatx4*>(p + 4);
+    f.v[0] = lo.x; f.v[1] = lo.y; f.v[2] = lo.z; f.v[3] = lo.w;
+    f.v[4] = hi.x; f.v[5] = hi.y; f.v[6] = hi.z; f.v[7] = hi.w;
+    return f;
+  }
+  __device__ static __forceinline__ frag from_floats(const float* p) {
+    frag f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f.v[j] = p[j];
+    return f;
+  }
+  __device__ static __forceinline__ void run(floatx16& c, const frag& a, const frag& b) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.v[j], b.v[j], c, 0, 0, 0);
+  }
+};
+
+// ------------------------------------------------------------------------------------------------
+// Prefill.  Everything is computed transposed so that one lane owns one query: S^T = K Q^T gives each
+// lane (query = lane % 32) sixteen keys of a 32-key tile, the online-softmax state is lane-local, and
+// O^T = V^T P^T is rescaled without any cross-lane traffic.  K rows are fetched in a permuted order so
+// that the sixteen keys a lane ends up with are 8 consecutive ones per MFMA k-step - exactly the
+// operand layout the second MFMA wants for P^T - and V comes pre-transposed ([dh][keys]).
+//
+// Workgroup: 4 wavefronts x 32 queries; K/V tiles of 32 keys staged through LDS.
+template <typename T, int DH>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ kc,
+                                                           const T* __restrict__ vt, const int32_t* __restrict__ pos0,
+                                                           int H, int Tp, int Tcap, int64_t ldvt, T* __restrict__ out,
+                                                           int64_t ld_out) {
+  constexpr int EPC = mma<T>::EPC;
+  using raw_t = typename mma<T>::raw_t;
+  constexpr int BKV = 32;
+  constexpr int KROW = DH + EPC;     // padded K row (elements)
+  constexpr int VROW = BKV + EPC;    // padded V^T row
+  constexpr int KS = DH / 16;        // MFMA k-steps over the head dim
+  constexpr int NBLK = DH / 32;      // 32-wide blocks of the head dim in O^T
+  __shared__ __align__(16) T Ks[BKV * KROW];
+  __shared__ __align__(16) T Vs[DH * VROW];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int fr = lane & 31, fg = lane >> 5;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int qt0 = blockIdx.x * 128;
+  const int p0 = pos0[b];                       // <= 0: minus the number of padding rows
+  const int t = qt0 + wave * 32 + fr;           // this lane's query (rectangle index)
+  const int qpos = (t < Tp) ? t + p0 : -1;      // its position; < 0 = padding / out of range
+  const int last_t = (qt0 + 127 < Tp - 1) ? qt0 + 127 : Tp - 1;
+  const int kmax = last_t + p0;                 // last key any query of this workgroup may see
+  const int klast = Tp - 1 + p0;                // last key position that exists for this sequence
+  const int64_t bh = (int64_t)b * H + h;
+
+  // Q fragments (B operand of S^T): lane (query fr, half fg) holds Q[t][ks*16 + fg*8 .. +8)
+  typename mma<T>::frag qf[KS];
+  {
+    const int tq = (t < Tp) ? t : Tp - 1;
+    const T* qp = q + (bh * Tp + tq) * DH + fg * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = mma<T>::load(qp + ks * 16);
+  }
+  // row fr of the S^T tile is key krow: rows {0-3, 4-7, 8-11, 12-15} <- keys {0-3, 8-11, 4-7, 12-15} (+16)
+  const int krow = 16 * (fr >> 4) + 8 * ((fr >> 2) & 1) + 4 * ((fr >> 3) & 1) + (fr & 3);
+
+  floatx16 o[NBLK];
+#pragma unroll
+  for (int i = 0; i < NBLK; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
+  float mrun = -INFINITY, lrun = 0.f;
+  const float scale = rsqrtf((float)DH);
+
+  const int ntiles = (kmax >= 0) ? kmax / BKV + 1 : 0;
+  for (int kt = 0; kt < ntiles; ++kt) {
+    const int key0 = kt * BKV;
+    __syncthreads();
+    // ---- stage K tile [32][DH] and V^T tile [DH][32]; keys that do not exist are zero-filled
+    {
+      constexpr int CPRK = DH / EPC;
+      for (int c = tid; c < BKV * CPRK; c += 256) {
+        const int row = c / CPRK, cc = c % CPRK;
+        const int key = key0 + row;
+        uint32x4 val = {0, 0, 0, 0};
+        if (key <= klast) val = *reinterpret_cast<const uint32x4*>(kc + (bh * Tcap + key) * DH + cc * EPC);
+        *reinterpret_cast<uint32x4*>(Ks + row * KROW + cc * EPC) = val;
+      }
+      constexpr int CPRV = BKV / EPC;
+      for (int c = tid; c < DH * CPRV; c += 256) {
+        const int row = c / CPRV, cc = c % CPRV;
+        const int key = key0 + cc * EPC;
+        uint32x4 val = {0, 0, 0, 0};
+        if (key + EPC - 1 <= klast) {
+          val = *reinterpret_cast<const uint32x4*>(vt + (bh * DH + row) * ldvt + key);
+        } else if (key <= klast) {
+          raw_t tmp[EPC];
+          const raw_t* vr = reinterpret_cast<const raw_t*>(vt) + (bh * DH + row) * ldvt + key;
+#pragma unroll
+          for (int j = 0; j < EPC; ++j) tmp[j] = (key + j <= klast) ? vr[j] : (raw_t)0;
+          val = *reinterpret_cast<uint32x4*>(tmp);
+        }
+        *reinterpret_cast<uint32x4*>(Vs + row * VROW + cc * EPC) = val;
+      }
+    }
+    __syncthreads();
+    // wave-uniform skip of tiles that lie entirely above this wavefront's last query
+    const int wave_last = qt0 + wave * 32 + 31 + p0;
+    if (key0 > wave_last) continue;
+
+    // ---- S^T tile: rows = (permuted) keys, columns = queries
+    floatx16 s;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+    {
+      const T* kp = Ks + krow * KROW + fg * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) mma<T>::run(s, mma<T>::load(kp + ks * 16), qf[ks]);
+    }
+    // register v of this lane is key key0 + 16*(v/8) + 8*fg + v%8
+    float p[16];
+    float mt = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = key0 + 16 * (v / 8) + 8 * fg + (v % 8);
+      const bool ok = key <= qpos;
+      p[v] = ok ? s[v] * scale : -INFINITY;
+      mt = fmaxf(mt, p[v]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 32));
+    const float mnew = fmaxf(mrun, mt);
+    const float msafe = (mnew == -INFINITY) ? 0.f : mnew;
+    const float alpha = expf(mrun - msafe);      // mrun = -inf -> 0
+    float lt = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      p[v] = expf(p[v] - msafe);                 // masked -> exp(-inf) = 0
+      lt += p[v];
+    }
+    lt += __shfl_xor(lt, 32);
+    lrun = lrun * alpha + lt;
+    mrun = mnew;
+#pragma unroll
+    for (int i = 0; i < NBLK; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
+
+    // ---- O^T += V^T P^T : A = V^T rows (head-dim), B = P^T (keys x queries)
+    const typename mma<T>::frag pf0 = mma<T>::from_floats(p), pf1 = mma<T>::from_floats(p + 8);
+#pragma unroll
+    for (int i = 0; i < NBLK; ++i) {
+      const T* vp = Vs + (i * 32 + fr) * VROW + fg * 8;
+      mma<T>::run(o[i], mma<T>::load(vp), pf0);
+      mma<T>::run(o[i], mma<T>::load(vp + 16), pf1);
+    }
+  }
+
+  // ---- write O: register v of block i is head-dim i*32 + 8*(v/4) + 4*fg + v%4 of query t
+  if (t < Tp) {
+    const float inv = (qpos >= 0 && lrun > 0.f) ? 1.0f / lrun : 0.f;
+    T* op = out + ((int64_t)b * Tp + t) * ld_out + (int64_t)h * DH;
+#pragma unroll
+    for (int i = 0; i < NBLK; ++i)
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const int e = i * 32 + 8 * v4 + 4 * fg;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) elem<T>::store(op + e + w, o[i][v4 * 4 + w] * inv);
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Decode.  Grid (splits, H, B); each workgroup reduces a contiguous range of window slots to a partial
+// (max, sum, weighted V) that attn_combine_kernel merges.  16-byte loads: LPK lanes cover one key row.
+template <typename T, int DH>
+__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const T* __restrict__ kc,
+                                                          const T* __restrict__ vc, const int32_t* __restrict__ pos,
+                                                          int H, int Tcap, int chunk, float* __restrict__ work) {
+  constexpr int EPC = 16 / sizeof(T);
+  constexpr int LPK = DH / EPC;      // lanes per key row
+  constexpr int KPL = 64 / LPK;      // keys per wavefront load
+  static_assert(LPK <= 64 && 64 % LPK == 0, "head dim does not map onto a wavefront");
+  extern __shared__ __align__(16) float sm[];   // [chunk] scores, then [4][DH] partial outputs
+  __shared__ float red[8];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z, S = gridDim.x;
+  const int64_t bh = (int64_t)b * H + h;
+  const int nvalid = (pos[b] + 1 < Tcap) ? pos[b] + 1 : Tcap;
+  const int k0 = split * chunk;
+  const int k1 = (k0 + chunk < nvalid) ? k0 + chunk : nvalid;
+  float* wout = work + (bh * S + split) * (DH + 2);
+  if (k1 <= k0) {  // empty range
+    for (int e = tid; e < DH; e += 256) wout[2 + e] = 0.f;
+    if (tid == 0) { wout[0] = -INFINITY; wout[1] = 0.f; }
+    return;
+  }
+  const int nk = k1 - k0;
+  const int sub = lane / LPK, el = (lane % LPK) * EPC;
+  float qv[EPC];
+#pragma unroll
+  for (int j = 0; j < EPC; ++j) qv[j] = q[bh * DH + el + j];
+  const float scale = rsqrtf((float)DH);
+
+  // ---- scores
+  const T* kbase = kc + (bh * Tcap + k0) * DH;
+  for (int kk = wave * KPL + sub; kk < nk + KPL; kk += 4 * KPL) {   // uniform trip count per wavefront
+    float d = 0.f;
+    if (kk < nk) {
+      const uint32x4 w = *reinterpret_cast<const uint32x4*>(kbase + (int64_t)kk * DH + el);
+      if (sizeof(T) == 2) {
+        d = bf16_lo(w.x) * qv[0] + bf16_hi(w.x) * qv[1 % EPC] + bf16_lo(w.y) * qv[2 % EPC] + bf16_hi(w.y) * qv[3 % EPC] +
+            bf16_lo(w.z) * qv[4 % EPC] + bf16_hi(w.z) * qv[5 % EPC] + bf16_lo(w.w) * qv[6 % EPC] + bf16_hi(w.w) * qv[7 % EPC];
+      } else {
+        d = __uint_as_float(w.x) * qv[0] + __uint_as_float(w.y) * qv[1] + __uint_as_float(w.z) * qv[2] +
+            __uint_as_float(w.w) * qv[3];
+      }
+    }
+#pragma unroll
+    for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o);
+    if (kk < nk && (lane % LPK) == 0) sm[kk] = d * scale;
+  }
+  __syncthreads();
+  // ---- softmax statistics of the range
+  float m = -INFINITY;
+  for (int i = tid; i < nk; i += 256) m = fmaxf(m, sm[i]);
+  m = wave_max(m);
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float l = 0.f;
+  for (int i = tid; i < nk; i += 256) {
+    const float p = expf(sm[i] - m);
+    sm[i] = p;
+    l += p;
+  }
+  l = wave_sum(l);
+  if (lane == 0) red[4 + wave] = l;
+  __syncthreads();
+  l = (red[4] + red[5]) + (red[6] + red[7]);
+
+  // ---- weighted V
+  float acc[EPC];
+#pragma unroll
+  for (int j = 0; j < EPC; ++j) acc[j] = 0.f;
+  const T* vbase = vc + (bh * Tcap + k0) * DH;
+  for (int kk = wave * KPL + sub; kk < nk; kk += 4 * KPL) {
+    const uint32x4 w = *reinterpret_cast<const uint32x4*>(vbase + (int64_t)kk * DH + el);
+    const float p = sm[kk];
+    if (sizeof(T) == 2) {
+      acc[0] += p * bf16_lo(w.x); acc[1 % EPC] += p * bf16_hi(w.x);
+      acc[2 % EPC] += p * bf16_lo(w.y); acc[3 % EPC] += p * bf16_hi(w.y);
+      acc[4 % EPC] += p * bf16_lo(w.z); acc[5 % EPC] += p * bf16_hi(w.z);
+      acc[6 % EPC] += p * bf16_lo(w.w); acc[7 % EPC] += p * bf16_hi(w.w);
+    } else {
+      acc[0] += p * __uint_as_float(w.x); acc[1] += p * __uint_as_float(w.y);
+      acc[2] += p * __uint_as_float(w.z); acc[3] += p * __uint_as_float(w.w);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < EPC; ++j)
+#pragma unroll
+    for (int o = 32; o >= LPK; o >>= 1) acc[j] += __shfl_xor(acc[j], o);
+  __syncthreads();                       // scores no longer needed: reuse sm as [4][DH]
+  if (lane < LPK)
+#pragma unroll
+    for (int j = 0; j < EPC; ++j) sm[wave * DH + el + j] = acc[j];
+  __syncthreads();
+  for (int e = tid; e < DH; e += 256) wout[2 + e] = (sm[e] + sm[DH + e]) + (sm[2 * DH + e] + sm[3 * DH + e]);
+  if (tid == 0) { wout[0] = m; wout[1] = l; }
+}
+
+template <int DH>
+__global__ void attn_combine_kernel(const float* __restrict__ work, int S, int H, void* __restrict__ out,
+                                    int64_t ld_out, int out_dtype) {
+  const int h = blockIdx.x, b = blockIdx.y, e = threadIdx.x;
+  const float* w = work + ((int64_t)b * H + h) * S * (DH + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < S; ++s) m = fmaxf(m, w[s * (DH + 2)]);
+  float l = 0.f, acc = 0.f;
+  for (int s = 0; s < S; ++s) {
+    const float f = expf(w[s * (DH + 2)] - m);
+    l += f * w[s * (DH + 2) + 1];
+    acc += f * w[s * (DH + 2) + 2 + e];
+  }
+  store_as(out, (int64_t)b * ld_out + h * DH + e, acc / l, out_dtype);
+}
+
+int decode_splits(int64_t B, int64_t H, int64_t Tcap) {
+  int64_t s = (1024 + B * H - 1) / (B * H);
+  const int64_t smax = (Tcap + 63) / 64;
+  if (s > smax) s = smax;
+  if (s < 1) s = 1;
+  return (int)s;
+}
+
+}  // namespace
+
+extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* v_t, const int32_t* pos0, int64_t B,
+                                int64_t H, int64_t Tp, int64_t Tcap, int64_t dh, int64_t ldvt, void* out,
+                                int64_t ld_out, int dtype, void* stream) {
+  MTJ_REQUIRE(q && k_cache && v_t && pos0 && out, MTJ_EINVAL, "mtj_attn_prefill: null pointer");
+  MTJ_REQUIRE(B > 0 && H > 0 && Tp > 0 && Tp <= Tcap && ld_out >= H * dh && B < 65536 && H < 65536, MTJ_EINVAL,
+              "mtj_attn_prefill: bad shape B=%lld H=%lld Tp=%lld Tcap=%lld", (long long)B, (long long)H,
+              (long long)Tp, (long long)Tcap);
+  const int esz = dtype == MTJ_BF16 ? 2 : 4;
+  MTJ_REQUIRE(ldvt >= Tp && (ldvt * esz) % 16 == 0 && (ld_out * esz) % 16 == 0, MTJ_EALIGN,
+              "mtj_attn_prefill: ldvt must be >= Tp and rows 16-byte aligned");
+  MTJ_REQUIRE(mtj_aligned16(q) && mtj_aligned16(k_cache) && mtj_aligned16(v_t) && mtj_aligned16(out), MTJ_EALIGN,
+              "mtj_attn_prefill: pointers must be 16-byte aligned");
+  dim3 grid((unsigned)((Tp + 127) / 128), (unsigned)H, (unsigned)B);
+  hipStream_t s = (hipStream_t)stream;
+#define MTJ_PREFILL(T, DH)                                                                                    \
+  attn_prefill_kernel<T, DH><<<grid, 256, 0, s>>>((const T*)q, (const T*)k_cache, (const T*)v_t, pos0, (int)H, \
+                                                  (int)Tp, (int)Tcap, ldvt, (T*)out, ld_out)
+  if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL(bf16_t, 256);
+  else if (dtype == MTJ_BF16 && dh == 64) MTJ_PREFILL(bf16_t, 64);
+  else if (dtype == MTJ_F32 && dh == 256) MTJ_PREFILL(float, 256);
+  else if (dtype == MTJ_F32 && dh == 64) MTJ_PREFILL(float, 64);
+  else return mtj_fail(MTJ_EINVAL, "mtj_attn_prefill: unsupported dtype %d / d_head %lld (64 or 256)", dtype, (long long)dh);
+#undef MTJ_PREFILL
+  return mtj_check_launch("mtj_attn_prefill");
+}
+
+extern "C" int64_t mtj_attn_decode_work_bytes(int64_t B, int64_t H, int64_t dh, int64_t Tcap) {
+  return B * H * (int64_t)decode_splits(B, H, Tcap) * (dh + 2) * (int64_t)sizeof(float);
+}
+
+extern "C" int mtj_attn_decode(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,
+                               int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
+                               void* work, void* stream) {
+  MTJ_REQUIRE(q && k_cache && v_cache && pos && out && work, MTJ_EINVAL, "mtj_attn_decode: null pointer");
+  MTJ_REQUIRE(B > 0 && H > 0 && Tcap > 0 && ld_out >= H * dh && B < 65536 && H < 65536, MTJ_EINVAL,
+              "mtj_attn_decode: bad shape");
+  MTJ_REQUIRE(out_dtype == MTJ_F32 || out_dtype == MTJ_BF16, MTJ_EDTYPE, "mtj_attn_decode: out_dtype %d", out_dtype);
+  MTJ_REQUIRE(mtj_aligned16(q) && mtj_aligned16(k_cache) && mtj_aligned16(v_cache), MTJ_EALIGN,
+              "mtj_attn_decode: pointers must be 16-byte aligned");
+  const int S = decode_splits(B, H, Tcap);
+  const int chunk = (int)((Tcap + S - 1) / S);
+  const size_t lds = sizeof(float) * (size_t)(chunk > 4 * dh ? chunk : 4 * dh);
+  MTJ_REQUIRE(lds <= 60 * 1024, MTJ_ELIMIT, "mtj_attn_decode: window chunk %d too large", chunk);
+  dim3 grid((unsigned)S, (unsigned)H, (unsigned)B);
+  hipStream_t s = (hipStream_t)stream;
+#define MTJ_DECODE(T, DH)                                                                                       \
+  do {                                                                                                          \
+    attn_decode_kernel<T, DH><<<grid, 256, lds, s>>>(q, (const T*)k_cache, (const T*)v_cache, pos, (int)H,      \
+                                                     (int)Tcap, chunk, (float*)work);                           \
+    attn_combine_kernel<DH><<<dim3((unsigned)H, (unsigned)B), DH, 0, s>>>((const float*)work, S, (int)H, out,   \
+                                                                          ld_out, out_dtype);                   \
+  } while (0)
+  if (dtype == MTJ_BF16 && dh == 256) MTJ_DECODE(bf16_t, 256);
+  else if (dtype == MTJ_BF16 && dh == 64) MTJ_DECODE(bf16_t, 64);
+  else if (dtype == MTJ_F32 && dh == 256) MTJ_DECODE(float, 256);
+  else if (dtype == MTJ_F32 && dh == 64) MTJ_DECODE(float, 64);
+  else return mtj_fail(MTJ_EINVAL, "mtj_attn_decode: unsupported dtype %d / d_head %lld (64 or 256)", dtype, (long long)dh);
+#undef MTJ_DECODE
+  return mtj_check_launch("mtj_attn_decode");
+}

@@ -1,0 +1,123 @@
+// Shared host/device helpers for the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include "mtj_abi.h"
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t uint32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t uint32x2 __attribute__((ext_vector_type(2)));
+
+#define MTJ_WAVE 64
+
+// ---------------------------------------------------------------- error plumbing (host)
+int mtj_fail(int code, const char* fmt, ...);
+int mtj_check_launch(const char* what);
+
+#define MTJ_REQUIRE(cond, code, ...) \
+  do {                               \
+    if (!(cond)) return mtj_fail(code, __VA_ARGS__); \
+  } while (0)
+
+static inline bool mtj_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---------------------------------------------------------------- device helpers
+// bf16 <-> f32.  Rounding to bf16 is round-to-nearest-even (what jnp.astype(bfloat16) does).
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t hi16) { return __uint_as_float(hi16 << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+template <typename T> struct elem;
+template <> struct elem<float> {
+  static constexpr int dtype = MTJ_F32;
+  __device__ static __forceinline__ float load(const float* p) { return *p; }
+  __device__ static __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <> struct elem<bf16_t> {
+  static constexpr int dtype = MTJ_BF16;
+  __device__ static __forceinline__ float load(const bf16_t* p) {
+    return bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(p));
+  }
+  __device__ static __forceinline__ void store(bf16_t* p, float v) {
+    *reinterpret_cast<uint16_t*>(p) = (uint16_t)f32_to_bf16_bits(v);
+  }
+};
+
+// store a float into a buffer whose element type is only known at run time
+__device__ __forceinline__ void store_as(void* base, int64_t idx, float v, int dtype) {
+  if (dtype == MTJ_F32) reinterpret_cast<float*>(base)[idx] = v;
+  else reinterpret_cast<uint16_t*>(base)[idx] = (uint16_t)f32_to_bf16_bits(v);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+
+// jax.nn.gelu(approximate=True): 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float c = 0.7978845608028654f;
+  float u = c * (x + 0.044715f * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(u));
+}
+
+// ---------------------------------------------------------------- fused input-projection epilogue
+// One output element (row m, column n) of q|v|k|fc_in.  `own` is the accumulator of column n,
+// `partner` the accumulator of column n ^ 1 of the same row (needed by the interleaved rotation,
+// layers.py:137-148: out[2i] = x[2i] cos - x[2i+1] sin, out[2i+1] = x[2i+1] cos + x[2i] sin).
+__device__ __forceinline__ void inproj_store(const mtj_inproj& ip, const float* __restrict__ b1, int kv_dtype,
+                                             int64_t m, int64_t n, float own, float partner) {
+  const int d = ip.n_heads * ip.d_head;
+  const int b = (int)(m / ip.Tp), t = (int)(m - (int64_t)b * ip.Tp);
+  const int pos = ip.pos0[b] + t;
+  if (n >= 3 * (int64_t)d) {  // fc_in -> gelu
+    const int64_t c = n - 3 * (int64_t)d;
+    const float g = gelu_tanh(own + b1[c]);
+    store_as(ip.act, m * ip.ld_act + d + c, g, ip.act_dtype);
+    return;
+  }
+  if (pos < 0) return;  // left padding: nothing reaches the cache
+  const int seg = (int)(n / d);          // 0 q, 1 v, 2 k
+  const int c = (int)(n - (int64_t)seg * d);
+  const int h = c / ip.d_head, e = c - h * ip.d_head;
+  float val = own;
+  if (seg != 1 && e < ip.rotary_dims) {
+    const int p = pos < ip.max_pos ? pos : ip.max_pos - 1;
+    const float sn = ip.sin_tab[(int64_t)p * (ip.rotary_dims / 2) + (e >> 1)];
+    const float cs = ip.cos_tab[(int64_t)p * (ip.rotary_dims / 2) + (e >> 1)];
+    val = (e & 1) ? (own * cs + partner * sn) : (own * cs - partner * sn);
+  }
+  if (seg == 0) {
+    const int64_t idx = (((int64_t)b * ip.n_heads + h) * ip.Tp + t) * ip.d_head + e;
+    store_as(ip.q, idx, val, ip.q_dtype);
+  } else {
+    const int slot = pos % ip.Tcap;
+    const int64_t idx = (((int64_t)b * ip.n_heads + h) * ip.Tcap + slot) * ip.d_head + e;
+    store_as(seg == 1 ? ip.v_cache : ip.k_cache, idx, val, kv_dtype);
+    if (seg == 1 && ip.v_t && pos < ip.ldvt) {  // transposed copy, indexed by position like the cache
+      const int64_t it = (((int64_t)b * ip.n_heads + h) * ip.d_head + e) * ip.ldvt + pos;
+      store_as(ip.v_t, it, val, kv_dtype);
+    }
+  }
+}

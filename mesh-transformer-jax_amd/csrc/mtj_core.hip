@@ -1,0 +1,160 @@
+// Error plumbing, weight packing, embedding gather and LayerNorm.
+#include "mtj_common.h"
+
+// ---------------------------------------------------------------- errors
+static thread_local char g_err[512] = "";
+
+int mtj_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int mtj_check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "%s: %s", what, hipGetErrorString(e));
+  return MTJ_OK;
+}
+
+extern "C" int mtj_version(void) { return MTJ_ABI_VERSION; }
+extern "C" const char* mtj_last_error(void) { return g_err; }
+
+// ---------------------------------------------------------------- pack: dst[(n_off+n)*Kt + k_off+k] = src[k*ld + n]
+// 32x32 tiles through LDS so that both the read (along n) and the write (along k) are coalesced.
+template <typename T>
+__global__ __launch_bounds__(256) void pack_kernel(const T* __restrict__ src, int64_t ld, int64_t K, int64_t N,
+                                                   T* __restrict__ dst, int64_t Kt, int64_t n_off, int64_t k_off) {
+  __shared__ T tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  const int64_t n0 = (int64_t)blockIdx.x * 32, k0 = (int64_t)blockIdx.y * 32;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t k = k0 + ty + i * 8, n = n0 + tx;
+    if (k < K && n < N) tile[ty + i * 8][tx] = src[k * ld + n];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t n = n0 + ty + i * 8, k = k0 + tx;
+    if (k < K && n < N) dst[(n_off + n) * Kt + k_off + k] = tile[tx][ty + i * 8];
+  }
+}
+
+extern "C" int mtj_pack_weight(const void* src, int64_t src_ld, int64_t K, int64_t N, void* dst, int64_t K_total,
+                               int64_t n_off, int64_t k_off, int dtype, void* stream) {
+  MTJ_REQUIRE(src && dst, MTJ_EINVAL, "mtj_pack_weight: null pointer");
+  MTJ_REQUIRE(K > 0 && N > 0 && src_ld >= N && n_off >= 0 && k_off >= 0 && k_off + K <= K_total, MTJ_EINVAL,
+              "mtj_pack_weight: bad shape K=%lld N=%lld ld=%lld K_total=%lld k_off=%lld", (long long)K, (long long)N,
+              (long long)src_ld, (long long)K_total, (long long)k_off);
+  dim3 grid((unsigned)((N + 31) / 32), (unsigned)((K + 31) / 32));
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == MTJ_F32)
+    pack_kernel<float><<<grid, 256, 0, s>>>((const float*)src, src_ld, K, N, (float*)dst, K_total, n_off, k_off);
+  else if (dtype == MTJ_BF16)
+    pack_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)src, src_ld, K, N, (uint16_t*)dst, K_total, n_off, k_off);
+  else
+    return mtj_fail(MTJ_EDTYPE, "mtj_pack_weight: dtype %d", dtype);
+  return mtj_check_launch("mtj_pack_weight");
+}
+
+// ---------------------------------------------------------------- embedding: one row per workgroup
+template <typename T>
+__global__ __launch_bounds__(256) void embed_kernel(const int32_t* __restrict__ tok, const T* __restrict__ W,
+                                                    const float* __restrict__ b, int64_t V, int64_t d,
+                                                    float* __restrict__ out) {
+  const int64_t m = blockIdx.x;
+  const int64_t t = (uint32_t)tok[m];
+  const bool hit = t < V;  // an out-of-range id is an all-zero one-hot row
+  for (int64_t c = threadIdx.x; c < d; c += blockDim.x) {
+    const float w = hit ? elem<T>::load(W + t * d + c) : 0.0f;
+    out[m * d + c] = w + b[c];
+  }
+}
+
+extern "C" int mtj_embed(const int32_t* tok, int64_t M, const void* W, const float* b, int64_t n_vocab, int64_t d,
+                         int dtype, float* out, void* stream) {
+  MTJ_REQUIRE(tok && W && b && out, MTJ_EINVAL, "mtj_embed: null pointer");
+  MTJ_REQUIRE(M > 0 && d > 0 && n_vocab > 0, MTJ_EINVAL, "mtj_embed: bad shape");
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == MTJ_F32)
+    embed_kernel<float><<<(unsigned)M, 256, 0, s>>>(tok, (const float*)W, b, n_vocab, d, out);
+  else if (dtype == MTJ_BF16)
+    embed_kernel<bf16_t><<<(unsigned)M, 256, 0, s>>>(tok, (const bf16_t*)W, b, n_vocab, d, out);
+  else
+    return mtj_fail(MTJ_EDTYPE, "mtj_embed: dtype %d", dtype);
+  return mtj_check_launch("mtj_embed");
+}
+
+// ---------------------------------------------------------------- LayerNorm: one wavefront per row
+// Two passes over a row that stays in registers (mean first, then centred variance, as the reference
+// computes jnp.var); all statistics float32.
+#define LN_MAX_PER_LANE 64  // d <= 64 * 64 * 4 = 16384
+
+template <int OUT_DTYPE>
+__global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ scale,
+                                                        const float* __restrict__ offset, int64_t M, int d,
+                                                        void* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const float* xr = x + row * d;
+  const int nvec = d >> 2;  // float4 chunks
+  floatx4 v[LN_MAX_PER_LANE / 4];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < LN_MAX_PER_LANE / 4; ++i) {
+    const int c = i * 64 + lane;
+    if (c < nvec) {
+      v[i] = *reinterpret_cast<const floatx4*>(xr + 4 * c);
+      sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+  }
+  const float mean = wave_sum(sum) / (float)d;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < LN_MAX_PER_LANE / 4; ++i) {
+    const int c = i * 64 + lane;
+    if (c < nvec) {
+      const floatx4 t = v[i] - mean;
+      sq += (t.x * t.x + t.y * t.y) + (t.z * t.z + t.w * t.w);
+    }
+  }
+  const float inv = rsqrtf(wave_sum(sq) / (float)d + 1e-5f);
+#pragma unroll
+  for (int i = 0; i < LN_MAX_PER_LANE / 4; ++i) {
+    const int c = i * 64 + lane;
+    if (c < nvec) {
+      const floatx4 sc = *reinterpret_cast<const floatx4*>(scale + 4 * c);
+      const floatx4 of = *reinterpret_cast<const floatx4*>(offset + 4 * c);
+      const floatx4 y = (sc * inv) * (v[i] - mean) + of;
+      if (OUT_DTYPE == MTJ_F32) {
+        *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(out) + row * d + 4 * c) = y;
+      } else {
+        uint32x2 p;
+        p.x = pack_bf16x2(y.x, y.y);
+        p.y = pack_bf16x2(y.z, y.w);
+        *reinterpret_cast<uint32x2*>(reinterpret_cast<uint16_t*>(out) + row * d + 4 * c) = p;
+      }
+    }
+  }
+}
+
+extern "C" int mtj_layernorm(const float* x, const float* scale, const float* offset, int64_t M, int64_t d,
+                             void* out, int out_dtype, void* stream) {
+  MTJ_REQUIRE(x && scale && offset && out, MTJ_EINVAL, "mtj_layernorm: null pointer");
+  MTJ_REQUIRE(M > 0 && d > 0 && d % 4 == 0 && d <= 64 * LN_MAX_PER_LANE, MTJ_EINVAL,
+              "mtj_layernorm: d=%lld must be a multiple of 4 and <= %d", (long long)d, 64 * LN_MAX_PER_LANE);
+  MTJ_REQUIRE(mtj_aligned16(x) && mtj_aligned16(scale) && mtj_aligned16(offset) && mtj_aligned16(out), MTJ_EALIGN,
+              "mtj_layernorm: pointers must be 16-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned grid = (unsigned)((M + 3) / 4);
+  if (out_dtype == MTJ_F32)
+    layernorm_kernel<MTJ_F32><<<grid, 256, 0, s>>>(x, scale, offset, M, (int)d, out);
+  else if (out_dtype == MTJ_BF16)
+    layernorm_kernel<MTJ_BF16><<<grid, 256, 0, s>>>(x, scale, offset, M, (int)d, out);
+  else
+    return mtj_fail(MTJ_EDTYPE, "mtj_layernorm: out_dtype %d", out_dtype);
+  return mtj_check_launch("mtj_layernorm");
+}

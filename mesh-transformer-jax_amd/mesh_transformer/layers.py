@@ -1,0 +1,165 @@
+"""Module-level surface of the reference's mesh_transformer/layers.py for the GPT-J path
+(ReplicatedLayerNorm, EmbeddingShard, TransformerLayerShard, ProjectionShard, rotary helpers), as thin
+wrappers over the HIP kernels so that every seam of the model can be compared on its own.
+
+The reference modules are haiku modules that pull their parameters from the enclosing transform; here
+each module is given the parameter tree explicitly (`params`, haiku names, leading shard axis of 1).
+Inputs and outputs are float32 CUDA tensors shaped like the reference's per-sequence arrays
+([tokens, d_model]); attn_bias must be 0 (only pe == "rotary" is on this path).
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import _abi
+from ._abi import EPI_STORE, F32, check, ptr
+from .engine import ROOT, Engine, _f32, rotary_tables
+
+
+def fixed_pos_embedding(x, seq_dim=0):
+    """layers.py:128-134: float64 sin/cos tables [n_pos, dim/2] for the last axis of x."""
+    dim = x.shape[-1]
+    inv_freq = 1.0 / (10000 ** (np.arange(0, dim, 2) / dim))
+    ang = np.einsum("i,j->ij", np.arange(x.shape[seq_dim]), inv_freq)
+    return np.sin(ang), np.cos(ang)
+
+
+def _dev(x):
+    if not torch.cuda.is_available():
+        raise RuntimeError("mesh_transformer.layers runs on an MI355X; no GPU is visible")
+    return x.device if isinstance(x, torch.Tensor) and x.is_cuda else torch.device("cuda:0")
+
+
+def _f32_in(x, dev):
+    return torch.as_tensor(x).to(dev, torch.float32).contiguous()
+
+
+class ReplicatedLayerNorm:
+    """layers.py:12-36."""
+
+    def __init__(self, offset=True, params=None):
+        self.offset = offset
+        self.params = params            # {"scale": [1, d], "offset": [1, d]}
+
+    def __call__(self, inputs):
+        L = _abi.lib()
+        dev = _dev(inputs)
+        x = _f32_in(inputs, dev)
+        d = x.shape[-1]
+        rows = x.reshape(-1, d)
+        scale = _f32(torch.as_tensor(self.params["scale"]).to(dev).reshape(-1))
+        off = _f32(torch.as_tensor(self.params["offset"]).to(dev).reshape(-1)) if self.offset else torch.zeros_like(scale)
+        out = torch.empty_like(rows)
+        with torch.cuda.device(dev):
+            check(L.mtj_layernorm(ptr(rows), ptr(scale), ptr(off), rows.shape[0], d, ptr(out), F32, _abi.stream_handle()))
+        return out.reshape(x.shape)
+
+
+class EmbeddingShard:
+    """layers.py:165-202 with pe == "rotary" (no positional table)."""
+
+    def __init__(self, config, params, name=None):
+        assert config["n_vocab"] % config.get("cores_per_replica", 1) == 0     # layers.py:172
+        self.config = config
+        p = params[ROOT + "embedding_shard/~/linear"]
+        self.w, self.b = p["w"], p["b"]
+
+    def __call__(self, x, dtype=None):
+        L = _abi.lib()
+        dev = _dev(self.w)
+        w = torch.as_tensor(self.w).to(dev)[0].contiguous()
+        b = _f32(torch.as_tensor(self.b).to(dev)[0])
+        tok = torch.as_tensor(np.asarray(x).astype(np.int32) if not isinstance(x, torch.Tensor) else x.to(torch.int32)).to(dev)
+        tok = tok.reshape(-1).contiguous()
+        out = torch.empty(tok.shape[0], w.shape[1], dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            check(L.mtj_embed(ptr(tok), tok.shape[0], ptr(w), ptr(b), w.shape[0], w.shape[1], _abi.dtype_code(w.dtype),
+                              ptr(out), _abi.stream_handle()))
+        return out
+
+
+class TransformerLayerShard:
+    """layers.py:229-366.  Returns the residual DELTA, like the reference; the caller adds x.
+
+    Decode state: {"k", "v": [1, H, Tcap, dh] device tensors in the weight dtype (k stored rotated,
+    slot = position % Tcap), "tokens_decoded": int}.  decode_once updates k and v IN PLACE (the reference
+    returns new arrays); the returned dict aliases the same tensors."""
+
+    def __init__(self, config, params, name="layer_0", init_scale=1.0, device="cuda:0"):
+        heads, dim = config["n_heads"], config["d_model"]
+        assert dim % heads == 0                                    # layers.py:238
+        assert heads % config.get("cores_per_replica", 1) == 0     # layers.py:239
+        self.config = config
+        self.index = int(name.split("_")[-1])
+        self.eng = Engine(config, params, device, layer_ids=[self.index], embed=False, proj=False)
+        self.dim, self.heads, self.dim_per_head = dim, heads, dim // heads
+        self.pe_rotary_dims = config.get("pe_rotary_dims", self.dim_per_head)
+
+    # ---- whole-layer entry points
+    def _prefill(self, x, given_length):
+        eng, w = self.eng, self.eng.w
+        x = _f32_in(x, eng.device)
+        T = x.shape[0]
+        with torch.cuda.device(eng.device):
+            ses = eng.session(1, max(T, 1), T, T + 1)
+            pad = T - int(given_length)
+            pos0 = torch.tensor([-pad], dtype=torch.int32, device=eng.device)
+            delta = torch.zeros(T, w.d, dtype=torch.float32, device=eng.device)
+            # the layer kernels add into a residual stream: run them on a copy and subtract
+            xs = x.clone()
+            eng.layer_prefill(ses, self.index, xs, ses.h_pf[:T], ses.act_pf[:T], T, pos0)
+            delta = xs - x
+        return delta, ses, pad
+
+    def __call__(self, x, attn_bias=0):
+        assert np.all(np.asarray(attn_bias) == 0), "attn_bias (T5 relative positions) is not on the GPT-J path"
+        delta, _, _ = self._prefill(x, x.shape[0])
+        return delta
+
+    def get_init_decode_state(self, x, given_length, attn_bias=0):
+        assert np.all(np.asarray(attn_bias) == 0)
+        delta, ses, pad = self._prefill(x, given_length)
+        T = x.shape[0]
+        # window of T slots; the given_length real tokens sit at positions 0 .. given_length-1
+        state = {"k": ses.kc[self.index], "v": ses.vc[self.index], "tokens_decoded": int(given_length), "_ses": ses}
+        return delta, state
+
+    def decode_once(self, decode_state, x, attn_bias=0):
+        assert np.all(np.asarray(attn_bias) == 0)
+        eng, w = self.eng, self.eng.w
+        x = _f32_in(x, eng.device)
+        assert x.shape[0] == 1                                     # layers.py:320
+        ses = decode_state["_ses"]
+        n = int(decode_state["tokens_decoded"])
+        with torch.cuda.device(eng.device):
+            if ses.max_pos <= n + 1:
+                ses.max_pos = 2 * (n + 1)
+                ses.sin, ses.cos = rotary_tables(ses.max_pos, eng.r, eng.device)
+            ses.pos.fill_(n)                                        # position of the new token
+            ses.x.copy_(x)
+            eng.layer_decode(ses, self.index)
+            delta = ses.x - x
+        return delta, {"k": ses.kc[self.index], "v": ses.vc[self.index], "tokens_decoded": n + 1, "_ses": ses}
+
+
+class ProjectionShard:
+    """layers.py:545-567: final LayerNorm + logits projection (the all_gather is the identity at one shard)."""
+
+    def __init__(self, config, params, name=None, device="cuda:0"):
+        assert config["n_vocab"] % config.get("cores_per_replica", 1) == 0     # layers.py:552
+        self.eng = Engine(config, params, device, layer_ids=[], embed=False, proj=True)
+
+    def __call__(self, x):
+        L = _abi.lib()
+        eng, w = self.eng, self.eng.w
+        x = _f32_in(x, eng.device).reshape(-1, w.d)
+        M = x.shape[0]
+        out = torch.empty(M, w.V, dtype=torch.float32, device=eng.device)
+        with torch.cuda.device(eng.device):
+            s = _abi.stream_handle()
+            h = torch.empty(M, w.d, dtype=w.torch_dtype, device=eng.device)
+            check(L.mtj_layernorm(ptr(x), ptr(w.pln_s), ptr(w.pln_o), M, w.d, ptr(h), w.dtype, s))
+            check(L.mtj_gemm(ptr(h), w.d, ptr(w.w_p), ptr(w.b_p), M, w.V, w.d, w.dtype, EPI_STORE, ptr(out), w.V, F32,
+                             None, s))
+        return out

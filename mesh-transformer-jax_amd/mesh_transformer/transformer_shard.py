@@ -1,0 +1,243 @@
+"""CausalTransformer with the call surface of the reference's mesh_transformer/transformer_shard.py
+(constructor from a config dict, .state["params"] in the haiku tree layout, .generate(...)), running
+on one MI355X through the HIP kernels.  Only the generate path exists here: train/eval/init_xmap,
+the xmap/pjit sharding and the optimizer state are not part of this build.
+"""
+import random
+
+import numpy as np
+import torch
+
+from . import _abi, sampling
+from .engine import ROOT, Engine
+
+
+def _init_tree(config, device, seed=42):
+    """Random-init parameter tree with haiku's shapes, names and initialisers
+    (transformer_shard.py:175-188, layers.py:180-185,249-258,559): hk.Linear weights are
+    TruncatedNormal(1/sqrt(fan_in)), out / fc_out use init_scale/sqrt(d_model) with
+    init_scale = 2/layers (transformer_shard.py:35), biases 0, LayerNorm scale 1 / offset 0.
+    "early_cast" in the config gives bfloat16 leaves (transformer_shard.py:185)."""
+    d, V, n = config["d_model"], config["n_vocab"], config["layers"]
+    F = 4 * d
+    dt = torch.bfloat16 if "early_cast" in config else torch.float32
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+
+    def tn(shape, std):
+        t = torch.empty(shape, dtype=torch.float32, device=device)
+        torch.nn.init.trunc_normal_(t, 0.0, std, -2 * std, 2 * std, generator=gen)
+        return t.to(dt)
+
+    zeros = lambda *s: torch.zeros(*s, dtype=dt, device=device)
+    ones = lambda *s: torch.ones(*s, dtype=dt, device=device)
+    tree = {ROOT + "embedding_shard/~/linear": {"w": tn((1, V, d), V ** -0.5), "b": zeros(1, d)}}
+    o_std = (2.0 / n) / d ** 0.5
+    for i in range(n):
+        p = f"{ROOT}layer_{i}/~/"
+        tree[p + "replicated_layer_norm"] = {"scale": ones(1, d), "offset": zeros(1, d)}
+        tree[p + "linear"] = {"w": tn((1, d, d), d ** -0.5)}       # q
+        tree[p + "linear_1"] = {"w": tn((1, d, d), d ** -0.5)}     # v
+        tree[p + "linear_2"] = {"w": tn((1, d, d), d ** -0.5)}     # k
+        tree[p + "linear_3"] = {"w": tn((1, d, d), o_std)}         # o
+        tree[p + "linear_4"] = {"w": tn((1, d, F), d ** -0.5), "b": zeros(1, F)}
+        tree[p + "linear_5"] = {"w": tn((1, F, d), o_std), "b": zeros(1, d)}
+    tree[ROOT + "projection_shard/~/replicated_layer_norm"] = {"scale": ones(1, d), "offset": zeros(1, d)}
+    tree[ROOT + "projection_shard/~/linear"] = {"w": tn((1, d, V), d ** -0.5), "b": zeros(1, V)}
+    return tree
+
+
+def _to_device_tree(tree, device):
+    out = {}
+    for mod, leaves in tree.items():
+        out[mod] = {k: torch.as_tensor(v).to(device) for k, v in leaves.items()}
+    return out
+
+
+class CausalTransformer:
+    """Drop-in for transformer_shard.py:118-339 on the generate path.
+
+    config keys read: layers, d_model, n_heads, n_vocab, norm, pe, pe_rotary_dims, cores_per_replica,
+    sampler (callable, transformer_shard.py:191), early_cast.  Extra, optional: "device",
+    "steps_per_graph" (decode steps recorded into one HIP graph, default 8; 0 disables graphs)."""
+
+    def __init__(self, config, params=None):
+        self.config = config
+        if config.get("cores_per_replica", 1) != 1:       # transformer_shard.py:257 asserts mp == cores_per_replica
+            raise ValueError("cores_per_replica must be 1: the model runs unsharded on one GPU")
+        if not torch.cuda.is_available():
+            raise RuntimeError("CausalTransformer needs an MI355X (HIP device); no GPU is visible")
+        _abi.lib()  # fail now, loudly, if the HIP library is not built
+        self.device = torch.device(config.get("device", "cuda:0"))
+        tree = _init_tree(config, self.device) if params is None else _to_device_tree(params, self.device)
+        self.state = {"params": tree, "step": np.array(0)}
+        self.gen_length = None
+        self.return_logits = False
+        self._engine = None
+        self._engine_key = None
+        n = sum(int(v.numel()) for m in tree.values() for v in m.values())
+        print(f"Total parameters: {n}")                  # transformer_shard.py:279-280
+
+    def from_params(self, tree):
+        """Replace the parameter tree (haiku names, leading shard axis of 1)."""
+        self.state = {"params": _to_device_tree(tree, self.device), "step": np.array(0)}
+        return self
+
+    def engine(self):
+        tree = self.state["params"]
+        key = tuple(v.data_ptr() for m in sorted(tree) for _, v in sorted(tree[m].items()))
+        if self._engine is None or key != self._engine_key:
+            self._engine = None
+            self._engine = Engine(self.config, tree, self.device)
+            self._engine_key = key
+        return self._engine
+
+    # ------------------------------------------------------------------ generate
+    def generate(self, ctx, ctx_length, gen_length, sampler_options, return_logits=False, uniforms=None,
+                 sampler=None, return_keep_mask=False):
+        """transformer_shard.py:326-339.
+
+        ctx uint32 [B, L] left-padded (device_sample.py:92-96), ctx_length [B], sampler_options a dict of
+        [B] arrays (top_p, temp, optional top_k).  Returns (final_state, (tokens [B, G, 1] uint32, None
+        [, logits [B, G, 1, V] float32])) so that callers' `out[1][0][:, :, 0]` works unchanged.
+
+        Beyond the reference: `uniforms` float64 [B, G] in [0, 1) drive the inverse-CDF draw (default:
+        drawn from an unseeded Philox stream, like the reference's unseeded key at :327);
+        `sampler` overrides config["sampler"]."""
+        eng = self.engine()
+        self.gen_length, self.return_logits = gen_length, return_logits
+        ctx = np.ascontiguousarray(np.asarray(ctx)).astype(np.int64)
+        if ctx.ndim != 2:
+            raise ValueError("ctx must be [batch, length]")
+        B, Lc = ctx.shape
+        P = np.asarray(ctx_length).astype(np.int64).reshape(-1)
+        if P.shape[0] != B:
+            raise ValueError("ctx_length must have one entry per sequence")
+        if Lc < 2 or P.min() < 1 or P.max() > Lc:
+            raise ValueError("need ctx length >= 2 and 1 <= ctx_length <= ctx length")
+        G = int(gen_length)
+        if G < 1:
+            raise ValueError("gen_length must be positive")
+        Tcap = Lc - 1                                    # K/V window = prefill length (layers.py:325-326)
+        Tp = int(P.max()) - 1                            # real prompt tokens that go through prefill
+        max_pos = int(P.max()) + G + 1
+        sampler = sampler if sampler is not None else self.config.get("sampler", sampling.nucleaus_sample)
+        kind = sampling.builtin_kind(sampler)
+
+        dev = self.device
+        with torch.cuda.device(dev):
+            ses = eng.session(B, Tcap, Tp, max_pos)
+            self._ensure_io(ses, G, eng.w.V)
+            # --- inputs
+            ses.pos0.copy_(torch.from_numpy((-(Tp - (P - 1))).astype(np.int32)))
+            ses.pos.copy_(torch.from_numpy((P - 1).astype(np.int32)))
+            ses.pos_start.copy_(ses.pos)
+            ses.tok.copy_(torch.from_numpy(ctx[:, -1].astype(np.int32)))
+            ses.out_tokens.zero_()
+            opts = dict(sampler_options or {})
+            if kind == "nucleus":
+                tp = np.broadcast_to(np.asarray(opts.get("top_p", 0.9), np.float64), (B,))
+                tm = np.broadcast_to(np.asarray(opts.get("temp", 1.0), np.float64), (B,))
+                ses.top_p.copy_(torch.from_numpy(np.array(tp)))
+                ses.temp.copy_(torch.from_numpy(np.array(tm)))
+                tk = opts.get("top_k", None)
+                ses.use_top_k = tk is not None
+                if ses.use_top_k:
+                    ses.top_k.copy_(torch.from_numpy(np.array(np.broadcast_to(np.asarray(tk, np.int32), (B,)))))
+                if uniforms is None:
+                    rng = np.random.Generator(np.random.Philox(random.randint(0, 2 ** 60)))
+                    uniforms = rng.random((B, G))
+                u = np.asarray(uniforms, np.float64)
+                if u.shape != (B, G):
+                    raise ValueError(f"uniforms must have shape {(B, G)}")
+                ses.uniforms[:, :G].copy_(torch.from_numpy(np.ascontiguousarray(u)))
+            # --- prefill
+            if Tp > 0:
+                rect = torch.from_numpy(np.ascontiguousarray(ctx[:, Lc - 1 - Tp:Lc - 1]).astype(np.int32)).to(dev)
+                eng.prefill(ses, rect, Tp)
+            # --- decode
+            logits_out = torch.empty(B, G, eng.w.V, dtype=torch.float32, device=dev) if return_logits else None
+            masks = torch.empty(G, B, eng.w.V, dtype=torch.uint8, device=dev) if return_keep_mask else None   # [step, row, V]
+            if kind is None:
+                self._decode_host_sampler(eng, ses, G, sampler, opts, logits_out)
+            else:
+                self._decode(eng, ses, G, kind, logits_out, masks)
+            torch.cuda.synchronize(dev)
+            toks = ses.out_tokens[:, :G].cpu().numpy().astype(np.uint32)[:, :, None]
+            final_state = (toks[:, -1], ses, None)
+            out = (toks, None)
+            if return_logits:
+                out = out + (logits_out.cpu().numpy()[:, :, None, :],)
+            if return_keep_mask:
+                out = out + (masks.permute(1, 0, 2).cpu().numpy().astype(bool),)
+            return final_state, out
+
+    def _ensure_io(self, ses, G, V):
+        if getattr(ses, "G_max", 0) < G:
+            dev = self.device
+            ses.G_max = max(G, 64)
+            ses.out_tokens = torch.zeros(ses.B, ses.G_max, dtype=torch.int32, device=dev)
+            ses.uniforms = torch.zeros(ses.B, ses.G_max, dtype=torch.float64, device=dev)
+            ses.top_p = torch.zeros(ses.B, dtype=torch.float64, device=dev)
+            ses.temp = torch.ones(ses.B, dtype=torch.float64, device=dev)
+            ses.top_k = torch.zeros(ses.B, dtype=torch.int32, device=dev)
+            ses.use_top_k = False
+            ses.graphs = {}
+
+    def _step(self, eng, ses, kind, keep_mask=None):
+        eng.decode_model(ses)
+        if kind == "greedy":
+            eng.sample_greedy(ses, ses.out_tokens)
+        else:
+            eng.sample_nucleus(ses, ses.out_tokens, ses.top_p, ses.temp, ses.top_k if ses.use_top_k else None,
+                               ses.uniforms, keep_mask=keep_mask)
+
+    def _decode(self, eng, ses, G, kind, logits_out, masks):
+        spg = int(self.config.get("steps_per_graph", 8))
+        eager = spg <= 0 or logits_out is not None or masks is not None
+        t = 0
+        while t < G:
+            if eager or t == 0:
+                # the first step always runs eagerly: it also performs the kernels' one-time setup
+                self._step(eng, ses, kind, None if masks is None else masks[t])
+                if logits_out is not None:
+                    logits_out[:, t].copy_(ses.logits)
+                t += 1
+                continue
+            n = spg if G - t >= spg else 1
+            self._graph(eng, ses, kind, n).replay()
+            t += n
+
+    def _graph(self, eng, ses, kind, n):
+        key = (kind, n, ses.use_top_k)
+        g = ses.graphs.get(key)
+        if g is None:
+            if kind == "nucleus" and ses.sample_work is None:
+                ses.sample_work = torch.empty(_abi.lib().mtj_sample_work_bytes(ses.B, eng.w.V), dtype=torch.uint8,
+                                              device=self.device)
+            torch.cuda.synchronize(self.device)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for _ in range(n):
+                    self._step(eng, ses, kind)
+            ses.graphs[key] = g
+        return g
+
+    def _decode_host_sampler(self, eng, ses, G, sampler, opts, logits_out):
+        """Any callable honouring the reference contract (transformer_shard.py:203):
+        sampler(key, logits[1, V], sampler_input, **options_of_this_sequence) -> (token[1], info)."""
+        B = ses.B
+        for t in range(G):
+            eng.decode_model(ses)
+            lg = ses.logits.cpu().numpy()
+            if logits_out is not None:
+                logits_out[:, t].copy_(ses.logits)
+            nxt = np.zeros(B, np.int32)
+            for b in range(B):
+                ob = {k: (None if v is None else np.asarray(v).reshape(-1)[b] if np.ndim(v) else v) for k, v in opts.items()}
+                tok, _ = sampler(None, lg[b:b + 1], np.uint32(0), **ob)
+                nxt[b] = int(np.asarray(tok).reshape(-1)[0])
+            nt = torch.from_numpy(nxt).to(self.device)
+            ses.tok.copy_(nt)
+            ses.out_tokens[:, t].copy_(nt)
+            ses.pos.add_(1)

@@ -1,0 +1,421 @@
+"""Kernel-level parity through the C ABI (ctypes) on a real MI355X.
+
+References are float64 evaluations of the same mathematics on the same (already rounded) inputs -
+torch on the host or device for plain linear algebra, the CPU oracle for everything that carries a
+convention of the reference (rotary interleaving, masks, window, sampler order)."""
+import ctypes as C
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import gptj_oracle as O
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def L():
+    from mesh_transformer import _abi
+    return _abi.lib()
+
+
+def abi():
+    from mesh_transformer import _abi
+    return _abi
+
+
+def S():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def rel_err(got, ref):
+    got, ref = got.double().cpu(), ref.double().cpu()
+    return float((got - ref).norm() / ref.norm().clamp_min(1e-30))
+
+
+def max_err(got, ref):
+    return float((got.double().cpu() - ref.double().cpu()).abs().max())
+
+
+TD = {"f32": torch.float32, "bf16": torch.bfloat16}
+# float32 path: the 1e-4 relative budget of the whole layer leaves ~1e-5 per kernel
+TOL = {"f32": 2e-6, "bf16": 6e-3}
+
+
+# ------------------------------------------------------------------ pack / embed / layernorm
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_pack_weight_transposes_with_offsets(L, dt):
+    a = abi()
+    g = torch.Generator().manual_seed(0)
+    K, N1, N2 = 96, 70, 40
+    w1 = torch.randn(K, N1, generator=g).to(TD[dt]).to(DEV)
+    w2 = torch.randn(K // 2, N2, generator=g).to(TD[dt]).to(DEV)
+    dst = torch.zeros(N1 + N2, K, dtype=TD[dt], device=DEV)
+    a.check(L.mtj_pack_weight(a.ptr(w1), N1, K, N1, a.ptr(dst), K, 0, 0, a.dtype_code(TD[dt]), S()))
+    a.check(L.mtj_pack_weight(a.ptr(w2), N2, K // 2, N2, a.ptr(dst), K, N1, K // 2, a.dtype_code(TD[dt]), S()))
+    torch.cuda.synchronize()
+    ref = torch.zeros_like(dst)
+    ref[:N1] = w1.T
+    ref[N1:, K // 2:] = w2.T
+    assert torch.equal(dst, ref)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_embed_is_row_gather_plus_bias(L, dt):
+    a = abi()
+    g = torch.Generator().manual_seed(1)
+    V, d = 1000, 512
+    W = (torch.randn(V, d, generator=g) * 0.02).to(TD[dt]).to(DEV)
+    b = (torch.randn(d, generator=g) * 0.02).to(DEV)
+    tok = torch.tensor([0, 999, 5, 5, 123], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, d, device=DEV)
+    a.check(L.mtj_embed(a.ptr(tok), 5, a.ptr(W), a.ptr(b), V, d, a.dtype_code(TD[dt]), a.ptr(out), S()))
+    torch.cuda.synchronize()
+    assert torch.equal(out, W[tok.long()].float() + b)      # one non-zero term per dot: exact
+
+
+@pytest.mark.parametrize("d", [512, 4096, 1024 + 4])
+@pytest.mark.parametrize("out_dt", ["f32", "bf16"])
+def test_layernorm(L, d, out_dt):
+    a = abi()
+    g = torch.Generator().manual_seed(2)
+    M = 37
+    x = (torch.randn(M, d, generator=g) * 3 + 1.5).to(DEV)
+    sc = (1 + 0.1 * torch.randn(d, generator=g)).to(DEV)
+    of = (0.1 * torch.randn(d, generator=g)).to(DEV)
+    out = torch.empty(M, d, dtype=TD[out_dt], device=DEV)
+    a.check(L.mtj_layernorm(a.ptr(x), a.ptr(sc), a.ptr(of), M, d, a.ptr(out), a.dtype_code(TD[out_dt]), S()))
+    torch.cuda.synchronize()
+    ref = O.replicated_layer_norm(x.double().cpu(), sc.double().cpu(), of.double().cpu())
+    assert rel_err(out, ref) < (2e-6 if out_dt == "f32" else 3e-3)
+    # a constant row gives exactly `offset`
+    xc = torch.full((1, d), 2.75, device=DEV)
+    o2 = torch.empty(1, d, device=DEV)
+    a.check(L.mtj_layernorm(a.ptr(xc), a.ptr(sc), a.ptr(of), 1, d, a.ptr(o2), 0, S()))
+    torch.cuda.synchronize()
+    assert torch.equal(o2[0], of)
+
+
+def test_layernorm_rejects_bad_shapes(L):
+    a = abi()
+    x = torch.zeros(2, 6, device=DEV)
+    with pytest.raises(ValueError):
+        a.check(L.mtj_layernorm(a.ptr(x), a.ptr(x), a.ptr(x), 2, 6, a.ptr(x), 0, S()))
+
+
+# ------------------------------------------------------------------ GEMM
+def _packed(w_haiku):
+    """haiku [K, N] -> packed [N, K] through the library."""
+    a = abi()
+    K, N = w_haiku.shape
+    dst = torch.empty(N, K, dtype=w_haiku.dtype, device=DEV)
+    a.check(abi().lib().mtj_pack_weight(a.ptr(w_haiku), N, K, N, a.ptr(dst), K, 0, 0, a.dtype_code(w_haiku.dtype), S()))
+    return dst
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (32, 256, 128), (33, 300, 192), (128, 128, 512), (200, 1000, 256),
+                                   (64, 520, 2560), (257, 96, 64)])
+def test_gemm_store_and_resid(L, dt, M, N, K):
+    a = abi()
+    g = torch.Generator().manual_seed(M * 7 + N)
+    A = torch.randn(M, K, generator=g).to(TD[dt]).to(DEV)
+    Wh = (torch.randn(K, N, generator=g) * 0.05).to(TD[dt]).to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    W = _packed(Wh)
+    ref = A.double() @ Wh.double() + bias.double()
+    out = torch.empty(M, N, device=DEV)
+    a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, a.dtype_code(TD[dt]), a.EPI_STORE, a.ptr(out), N, 0,
+                       None, S()))
+    torch.cuda.synchronize()
+    assert rel_err(out, ref) < 5e-6, (dt, M, N, K)      # inputs are already rounded: only fp32 accumulation differs
+    # RESID: x += A W + b, with a padded leading dimension
+    x0 = torch.randn(M, N + 8, generator=g).to(DEV)
+    x = x0.clone()
+    a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, a.dtype_code(TD[dt]), a.EPI_RESID, a.ptr(x), N + 8, 0,
+                       None, S()))
+    torch.cuda.synchronize()
+    assert rel_err(x[:, :N], x0[:, :N].double() + ref) < 5e-6
+    assert torch.equal(x[:, N:], x0[:, N:])
+    # bf16 output
+    ob = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), None, M, N, K, a.dtype_code(TD[dt]), a.EPI_STORE, a.ptr(ob), N, 1, None, S()))
+    torch.cuda.synchronize()
+    assert rel_err(ob, A.double() @ Wh.double()) < 3e-3
+
+
+def test_gemm_rejects_bad_arguments(L):
+    a = abi()
+    A = torch.zeros(4, 48, device=DEV)
+    with pytest.raises(ValueError):   # K not a multiple of the k-tile
+        a.check(L.mtj_gemm(a.ptr(A), 48, a.ptr(A), None, 4, 4, 48, 0, a.EPI_STORE, a.ptr(A), 4, 0, None, S()))
+    with pytest.raises(ValueError):   # INPROJ without geometry
+        a.check(L.mtj_gemm(a.ptr(A), 32, a.ptr(A), None, 4, 4, 32, 0, a.EPI_INPROJ, None, 0, 0, None, S()))
+
+
+# ------------------------------------------------------------------ GEMV
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("N,K", [(512, 256), (28672, 4096), (4096, 20480), (50400, 4096), (514, 2560), (6, 520)])
+def test_gemv_store_resid_and_layernorm(L, dt, N, K):
+    a = abi()
+    g = torch.Generator().manual_seed(N + K)
+    x = torch.randn(K, generator=g).to(DEV)
+    Wh = (torch.randn(K, N, generator=g) * 0.02).to(TD[dt]).to(DEV)
+    W = _packed(Wh)
+    bias = torch.randn(N, generator=g).to(DEV)
+    ref = x.double() @ Wh.double() + bias.double()
+    out = torch.empty(N, device=DEV)
+    a.check(L.mtj_gemv(a.ptr(x), None, None, a.ptr(W), a.ptr(bias), N, K, a.dtype_code(TD[dt]), a.EPI_STORE, a.ptr(out), 0,
+                       None, S()))
+    torch.cuda.synchronize()
+    assert rel_err(out, ref) < 5e-6
+    y0 = torch.randn(N, generator=g).to(DEV)
+    y = y0.clone()
+    a.check(L.mtj_gemv(a.ptr(x), None, None, a.ptr(W), a.ptr(bias), N, K, a.dtype_code(TD[dt]), a.EPI_RESID, a.ptr(y), 0,
+                       None, S()))
+    torch.cuda.synchronize()
+    assert rel_err(y, y0.double() + ref) < 5e-6
+    if K <= 16384:
+        sc = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+        of = (0.1 * torch.randn(K, generator=g)).to(DEV)
+        xr = (x * 2 + 0.7)
+        a.check(L.mtj_gemv(a.ptr(xr), a.ptr(sc), a.ptr(of), a.ptr(W), a.ptr(bias), N, K, a.dtype_code(TD[dt]), a.EPI_STORE,
+                           a.ptr(out), 0, None, S()))
+        torch.cuda.synchronize()
+        h = O.replicated_layer_norm(xr.double().cpu()[None], sc.double().cpu(), of.double().cpu())[0].to(DEV)
+        assert rel_err(out, h @ Wh.double() + bias.double()) < 6e-6
+
+
+# ------------------------------------------------------------------ fused input projection (GEMM and GEMV)
+def _layer_params(cfg, seed, dt):
+    p = O.seeded_params(cfg, seed, TD[dt])
+    return p
+
+
+def _inproj_reference(cfg, p, x64, positions):
+    """q (rotated), k (rotated), v, gelu(fc_in) of layer 0 for rows at the given absolute positions (float64)."""
+    l = O.Layer(cfg, p, 0, torch.float64)
+    h = l.norm(x64)
+    q, v, k = l.qvk_proj(h)
+    r = l.r
+    sin, cos = O.fixed_pos_embedding(int(max(positions)) + 1, r)
+    sin, cos = sin[positions], cos[positions]
+
+    def rot(t):
+        tr = t[:, :, :r]
+        s = torch.as_tensor(sin).repeat_interleave(2, -1)[:, None, :]
+        c = torch.as_tensor(cos).repeat_interleave(2, -1)[:, None, :]
+        return torch.cat([tr * c + O.rotate_every_two(tr) * s, t[:, :, r:]], -1)
+
+    return rot(q), rot(k), v, O.gelu_tanh(h @ l.w1 + l.b1), h
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("shape", ["tiny", "head256"])
+def test_inproj_gemm_prefill_with_left_padding(dt, shape):
+    from mesh_transformer.engine import Engine
+    a = abi()
+    cfg = dict(layers=1, d_model=512, n_heads=8, n_vocab=64, pe="rotary", pe_rotary_dims=32, cores_per_replica=1) \
+        if shape == "tiny" else \
+        dict(layers=1, d_model=512, n_heads=2, n_vocab=64, pe="rotary", pe_rotary_dims=64, cores_per_replica=1)
+    p = _layer_params(cfg, 3, dt)
+    eng = Engine(cfg, {k: {n: v.to(DEV) for n, v in m.items()} for k, m in p.items()}, DEV, layer_ids=[0], embed=False, proj=False)
+    B, Tp, Tcap = 2, 40, 50
+    pads = [0, 7]
+    ses = eng.session(B, Tcap, Tp, 64)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(B * Tp, 512, generator=g).to(DEV)
+    pos0 = torch.tensor([-pd for pd in pads], dtype=torch.int32, device=DEV)
+    w = eng.w
+    L = a.lib()
+    h = ses.h_pf[:B * Tp]
+    act = ses.act_pf[:B * Tp]
+    a.check(L.mtj_layernorm(a.ptr(x), a.ptr(w.ln_s[0]), a.ptr(w.ln_o[0]), B * Tp, 512, a.ptr(h), w.dtype, S()))
+    ip = eng._inproj(ses, 0, Tp, pos0, ses.q_pf, w.dtype, act, w.dtype, ses.vt)
+    a.check(L.mtj_gemm(a.ptr(h), 512, a.ptr(w.w_in[0]), a.ptr(w.b1[0]), B * Tp, 3 * 512 + 2048, 512, w.dtype, a.EPI_INPROJ,
+                       None, 0, 0, C.byref(ip), S()))
+    torch.cuda.synchronize()
+    H, dh = eng.H, eng.dh
+    tol = TOL[dt] * (3 if dt == "f32" else 1.5)
+    for b in range(B):
+        pd = pads[b]
+        rows = x[b * Tp + pd:(b + 1) * Tp].double().cpu()
+        positions = np.arange(Tp - pd)
+        q_ref, k_ref, v_ref, g_ref, _ = _inproj_reference(cfg, p, rows, positions)
+        q = ses.q_pf[:B * H * Tp * dh].reshape(B, H, Tp, dh)[b, :, pd:].permute(1, 0, 2)
+        assert rel_err(q, q_ref) < tol
+        kk = ses.kc[0][b, :, :Tp - pd].permute(1, 0, 2)
+        vv = ses.vc[0][b, :, :Tp - pd].permute(1, 0, 2)
+        assert rel_err(kk, k_ref) < tol and rel_err(vv, v_ref) < tol
+        vt = ses.vt.reshape(B, H, dh, ses.ldvt)[b, :, :, :Tp - pd].permute(2, 0, 1)
+        assert torch.equal(vt.contiguous(), vv.contiguous())
+        assert rel_err(act[b * Tp + pd:(b + 1) * Tp, 512:], g_ref) < tol
+        # nothing was written for padding rows: the slots after the real tokens are still zero
+        assert float(ses.kc[0][b, :, Tp - pd:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_inproj_gemv_decode_appends_to_ring(dt):
+    from mesh_transformer.engine import Engine
+    a = abi()
+    cfg = dict(layers=1, d_model=512, n_heads=8, n_vocab=64, pe="rotary", pe_rotary_dims=32, cores_per_replica=1)
+    p = _layer_params(cfg, 5, dt)
+    eng = Engine(cfg, {k: {n: v.to(DEV) for n, v in m.items()} for k, m in p.items()}, DEV, layer_ids=[0], embed=False, proj=False)
+    Tcap = 6
+    ses = eng.session(1, Tcap, 1, 64)
+    L, w = a.lib(), eng.w
+    g = torch.Generator().manual_seed(6)
+    for pos in (0, 5, 6, 13):            # 6 and 13 wrap around the 6-slot window
+        x = torch.randn(1, 512, generator=g).to(DEV)
+        ses.pos.fill_(pos)
+        ip = eng._inproj(ses, 0, 1, ses.pos, ses.q, 0, ses.act, 0, None)
+        a.check(L.mtj_gemv(a.ptr(x), a.ptr(w.ln_s[0]), a.ptr(w.ln_o[0]), a.ptr(w.w_in[0]), a.ptr(w.b1[0]), 3 * 512 + 2048, 512,
+                           w.dtype, a.EPI_INPROJ, None, 0, C.byref(ip), S()))
+        torch.cuda.synchronize()
+        q_ref, k_ref, v_ref, g_ref, _ = _inproj_reference(cfg, p, x.double().cpu(), np.array([pos]))
+        tol = TOL[dt] * 3 if dt == "f32" else 5e-3
+        assert rel_err(ses.q.reshape(1, eng.H, eng.dh), q_ref) < 3e-6
+        assert rel_err(ses.kc[0][0, :, pos % Tcap][None], k_ref) < tol
+        assert rel_err(ses.vc[0][0, :, pos % Tcap][None], v_ref) < tol
+        assert rel_err(ses.act[:, 512:], g_ref) < 3e-6
+
+
+# ------------------------------------------------------------------ attention
+def _attn_reference(q, k, v, n_pad):
+    """q, k, v: [T, H, dh] float64, already rotated; causal + left-pad mask; returns [T - n_pad, H*dh]."""
+    T, H, dh = q.shape
+    s = torch.einsum("thd,Thd->htT", q, k) / math.sqrt(dh)
+    bias = O.MASK * (1.0 - torch.tril(torch.ones(T, T, dtype=torch.float64)))
+    bias = bias - 1e10 * (torch.arange(T) < n_pad).double()
+    w = torch.softmax(s + bias, -1)
+    return torch.einsum("htT,Thd->thd", w, v).reshape(T, H * dh)[n_pad:]
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("dh,H", [(64, 3), (256, 2)])
+@pytest.mark.parametrize("Tp", [1, 33, 128, 200])
+def test_attn_prefill(L, dt, dh, H, Tp):
+    a = abi()
+    g = torch.Generator().manual_seed(Tp + dh)
+    B, Tcap = 2, Tp + 3
+    pads = [0, min(5, Tp - 1)]
+    ldvt = (Tp + 31) // 32 * 32
+    q = torch.randn(B, H, Tp, dh, generator=g).to(TD[dt]).to(DEV)
+    kc = torch.zeros(B, H, Tcap, dh, dtype=TD[dt], device=DEV)
+    vt = torch.full((B, H, dh, ldvt), float("nan"), dtype=TD[dt], device=DEV)   # unwritten keys must never be read
+    kk = torch.randn(B, H, Tp, dh, generator=g).to(TD[dt]).to(DEV)
+    vv = torch.randn(B, H, Tp, dh, generator=g).to(TD[dt]).to(DEV)
+    for b in range(B):
+        n = Tp - pads[b]
+        kc[b, :, :n] = kk[b, :, pads[b]:]
+        vt[b, :, :, :n] = vv[b, :, pads[b]:].permute(0, 2, 1)
+    pos0 = torch.tensor([-pd for pd in pads], dtype=torch.int32, device=DEV)
+    ld_out = H * dh + 16
+    out = torch.full((B * Tp, ld_out), 7.0, dtype=TD[dt], device=DEV)
+    a.check(L.mtj_attn_prefill(a.ptr(q), a.ptr(kc), a.ptr(vt), a.ptr(pos0), B, H, Tp, Tcap, dh, ldvt, a.ptr(out), ld_out,
+                               a.dtype_code(TD[dt]), S()))
+    torch.cuda.synchronize()
+    for b in range(B):
+        pd = pads[b]
+        ref = _attn_reference(q[b].permute(1, 0, 2).double().cpu(), kk[b].permute(1, 0, 2).double().cpu(),
+                              vv[b].permute(1, 0, 2).double().cpu(), pd)
+        got = out[b * Tp + pd:(b + 1) * Tp, :H * dh]
+        assert rel_err(got, ref) < (3e-6 if dt == "f32" else 8e-3), (dt, dh, Tp, b)
+        assert float(out[b * Tp:b * Tp + pd, :H * dh].float().abs().max() if pd else 0.0) == 0.0   # padding rows: zeros
+    assert torch.all(out[:, H * dh:] == 7.0)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("dh,H", [(64, 8), (256, 16)])
+@pytest.mark.parametrize("Tcap,positions", [(7, [0, 6, 9]), (300, [0, 150, 299]), (2047, [511, 2046, 5000])])
+def test_attn_decode_window(L, dt, dh, H, Tcap, positions):
+    a = abi()
+    g = torch.Generator().manual_seed(Tcap + dh)
+    B = len(positions)
+    q = torch.randn(B, H, dh, generator=g).to(DEV)
+    kc = torch.randn(B, H, Tcap, dh, generator=g).to(TD[dt]).to(DEV)
+    vc = torch.randn(B, H, Tcap, dh, generator=g).to(TD[dt]).to(DEV)
+    pos = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    work = torch.empty(L.mtj_attn_decode_work_bytes(B, H, dh, Tcap), dtype=torch.uint8, device=DEV)
+    out = torch.zeros(B, H * dh + 8, device=DEV)
+    a.check(L.mtj_attn_decode(a.ptr(q), a.ptr(kc), a.ptr(vc), a.ptr(pos), B, H, Tcap, dh, a.ptr(out), H * dh + 8, 0,
+                              a.dtype_code(TD[dt]), a.ptr(work), S()))
+    torch.cuda.synchronize()
+    for b, p in enumerate(positions):
+        n = min(p + 1, Tcap)
+        s = torch.einsum("hd,hTd->hT", q[b].double(), kc[b, :, :n].double()) / math.sqrt(dh)
+        ref = torch.einsum("hT,hTd->hd", torch.softmax(s, -1), vc[b, :, :n].double()).reshape(-1)
+        assert rel_err(out[b, :H * dh], ref) < 3e-6, (dt, dh, Tcap, p)
+
+
+# ------------------------------------------------------------------ samplers: bit-exact against the oracle
+def _sample(L, logits, top_p, temp, top_k, u):
+    a = abi()
+    R, V = logits.shape
+    lg = torch.from_numpy(logits).to(DEV)
+    f64 = lambda v: torch.tensor(np.broadcast_to(np.asarray(v, np.float64), (R,)).copy(), dtype=torch.float64, device=DEV)
+    tk = None if top_k is None else torch.tensor(np.broadcast_to(np.asarray(top_k, np.int32), (R,)).copy(), dtype=torch.int32, device=DEV)
+    uu = f64(u).reshape(R, 1).contiguous()
+    tok = torch.zeros(R, dtype=torch.int32, device=DEV)
+    pos = torch.zeros(R, dtype=torch.int32, device=DEV)
+    pos_start = torch.zeros(R, dtype=torch.int32, device=DEV)
+    mask = torch.zeros(R, V, dtype=torch.uint8, device=DEV)
+    filt = torch.zeros(R, V, dtype=torch.float32, device=DEV)
+    work = torch.empty(L.mtj_sample_work_bytes(R, V), dtype=torch.uint8, device=DEV)
+    tp, tm = f64(top_p), f64(temp)
+    a.check(L.mtj_sample_nucleus(a.ptr(lg), R, V, a.ptr(tp), a.ptr(tm), a.ptr(tk), a.ptr(uu), 1, a.ptr(tok), None, 0,
+                                 a.ptr(pos), a.ptr(pos_start), a.ptr(mask), a.ptr(filt), a.ptr(work), S()))
+    torch.cuda.synchronize()
+    assert torch.all(pos == 1)
+    return tok.cpu().numpy(), mask.cpu().numpy().astype(bool), filt.cpu().numpy()
+
+
+def test_nucleus_reference_demo_vector(L):
+    demo = np.array([[-2, -1, 0, 0.8, 0, 0.1, 0.3, 0.4, 0.5, 0.6, 0.7, -3]], np.float32)   # sampling.py:49
+    tok, mask, filt = _sample(L, demo, 0.9, 1.0, None, 0.5)
+    assert set(np.nonzero(~mask[0])[0].tolist()) == {0, 1, 11}
+    assert np.array_equal(filt, O.nucleaus_filter(demo, 0.9))
+
+
+@pytest.mark.parametrize("V", [12, 1000, 50400])
+@pytest.mark.parametrize("spread", [0.3, 1.3, 6.0])
+def test_nucleus_bit_exact_vs_oracle(L, V, spread):
+    rng = np.random.default_rng(V + int(spread * 10))
+    R = 6
+    logits = (rng.standard_normal((R, V)) * spread).astype(np.float32)
+    logits[1, : V // 2] = logits[1, V // 2: 2 * (V // 2)]        # a row full of ties
+    logits[2, 3] = -0.0
+    logits[2, 4] = 0.0
+    top_p = np.array([0.9, 0.5, 0.999, 0.05, 1.0, 0.7])
+    temp = np.array([0.8, 1.0, 1.5, 0.3, 0.8, 2.0])
+    u = rng.random(R)
+    for top_k in (None, np.array([40, 1, 5, V, 3, 100], np.int32)):
+        tok, mask, filt = _sample(L, logits, top_p, temp, top_k, u)
+        for r in range(R):
+            k = None if top_k is None else int(top_k[r])
+            f_ref = O.nucleaus_filter(logits[r:r + 1], float(top_p[r]), k)
+            assert np.array_equal(filt[r:r + 1], f_ref), (V, spread, r, k)
+            assert np.array_equal(mask[r], f_ref[0] == logits[r])
+            assert tok[r] == O.inverse_cdf_draw(logits[r:r + 1], f_ref, float(temp[r]), float(u[r])), (V, spread, r, k)
+
+
+def test_greedy_lowest_index_on_ties(L):
+    a = abi()
+    V = 50400
+    lg = torch.zeros(3, V, device=DEV)
+    lg[0, 777] = 2.0
+    lg[0, 40000] = 2.0
+    lg[1, V - 1] = 1.0
+    tok = torch.zeros(3, dtype=torch.int32, device=DEV)
+    pos = torch.tensor([4, 5, 6], dtype=torch.int32, device=DEV)
+    pos_start = torch.tensor([4, 4, 4], dtype=torch.int32, device=DEV)
+    out = torch.full((3, 4), -1, dtype=torch.int32, device=DEV)
+    a.check(L.mtj_sample_greedy(a.ptr(lg), 3, V, a.ptr(tok), a.ptr(out), 4, a.ptr(pos), a.ptr(pos_start), S()))
+    torch.cuda.synchronize()
+    assert tok.tolist() == [777, V - 1, 0]
+    assert out.tolist() == [[777, -1, -1, -1], [-1, V - 1, -1, -1], [-1, -1, 0, -1]]
+    assert pos.tolist() == [5, 6, 7]

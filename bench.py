@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPT-J-6B generate path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+
+A "step" is one batch-1 greedy decode step of GPT-J-6B (bf16 weights, random init) after a 512-token
+prompt left-padded to 2048 (BASELINE config 3).  W untimed steps, then exactly K steps between two
+device synchronisations.  Prints ONE JSON line; `value` is generated tokens per second.
+
+Also reported on the same line:
+  roofline      the dominant kernel (the fused LayerNorm + q|v|k|fc_in GEMV, 28 launches per step):
+                algorithmic bytes of one launch / its average duration (HIP events), against 8 TB/s
+  step_hbm      whole-step algorithmic bytes / measured step time
+  prefill       the 511-token prefill of the same run, and one full-shape layer at [8 x 2048] tokens
+                (BASELINE config 2), as TFLOP/s against the 2.5 PFLOP/s bf16 MFMA peak
+  cpu_baseline  the CPU oracle (torch float32 on the host cores) on a bounded sample of the workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "mesh-transformer-jax_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK = 8.0e12          # B/s
+MFMA_BF16_PEAK = 2.5e15    # flop/s dense
+
+CFG_6B = dict(layers=28, d_model=4096, n_heads=16, n_vocab=50400, norm="layernorm", pe="rotary", pe_rotary_dims=64,
+              seq=2048, cores_per_replica=1, early_cast=True)
+
+
+def synthetic_tree(cfg, seed, device, dtype, std=0.02):
+    """Random-init tree: every weight and bias ~ N(0, 0.02), LayerNorm scale 1 / offset 0."""
+    import torch
+    from mesh_transformer.engine import ROOT as R
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    d, V, F = cfg["d_model"], cfg["n_vocab"], 4 * cfg["d_model"]
+    rn = lambda *s: (torch.randn(*s, generator=g, device=device, dtype=torch.float32) * std).to(dtype)
+    ln = lambda: {"scale": torch.ones(1, d, dtype=dtype, device=device), "offset": torch.zeros(1, d, dtype=dtype, device=device)}
+    t = {R + "embedding_shard/~/linear": {"w": rn(1, V, d), "b": rn(1, d)}}
+    for i in range(cfg["layers"]):
+        p = f"{R}layer_{i}/~/"
+        t[p + "replicated_layer_norm"] = ln()
+        for name in ("linear", "linear_1", "linear_2", "linear_3"):
+            t[p + name] = {"w": rn(1, d, d)}
+        t[p + "linear_4"] = {"w": rn(1, d, F), "b": rn(1, F)}
+        t[p + "linear_5"] = {"w": rn(1, F, d), "b": rn(1, d)}
+    t[R + "projection_shard/~/replicated_layer_norm"] = ln()
+    t[R + "projection_shard/~/linear"] = {"w": rn(1, d, V), "b": rn(1, V)}
+    return t
+
+
+def decode_bytes_per_step(cfg, ctx_mean, B=1):
+    """Algorithmic HBM bytes of one decode step: every weight once, K/V window read + one slot written,
+    embedding rows, logits."""
+    d, V, n, F = cfg["d_model"], cfg["n_vocab"], cfg["layers"], 4 * cfg["d_model"]
+    layer = (4 * d * d + 2 * d * F) * 2 + (F + d + 2 * d) * 2          # bf16 matrices + biases/LN as stored
+    weights = n * layer + (d * V + V + 2 * d) * 2
+    kv = B * n * 2 * d * 2 * (ctx_mean + 1)
+    return weights + kv + B * d * 2 + B * V * 4
+
+
+def gemv_inproj_bytes(cfg):
+    d, F = cfg["d_model"], 4 * cfg["d_model"]
+    return (3 * d + F) * d * 2 + d * 4 + 2 * d * 4 + F * 4 + (3 * d + F) * 4   # W_in + x + LN params + b1 + outputs
+
+
+def time_dominant_kernel(net, ses, reps=20):
+    """Average duration of the fused LayerNorm + q|v|k|fc_in GEMV, measured with HIP events on the stream it is
+    launched on: 28 back-to-back launches (one per layer, 6.6 GB of distinct weights, so nothing is re-read
+    from cache) per repetition."""
+    import ctypes as C
+    import torch
+    from mesh_transformer import _abi
+    from mesh_transformer._abi import EPI_INPROJ, F32, check, ptr
+    eng = net.engine()
+    L, w = _abi.lib(), eng.w
+    d, F = w.d, w.F
+    s = _abi.stream_handle()
+    ses.pos.fill_(600)
+    ses.x.normal_()
+
+    def sweep():
+        for i in w.layer_ids:
+            ip = eng._inproj(ses, i, 1, ses.pos, ses.q, F32, ses.act, F32, None)
+            check(L.mtj_gemv(ptr(ses.x), ptr(w.ln_s[i]), ptr(w.ln_o[i]), ptr(w.w_in[i]), ptr(w.b1[i]), 3 * d + F, d,
+                             w.dtype, EPI_INPROJ, None, 0, C.byref(ip), s))
+
+    sweep()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        sweep()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e-3 / (reps * len(w.layer_ids))
+
+
+def time_prefill_layer(net, B=8, T=2048, reps=5):
+    """One full-shape layer forward on [B x T] tokens (BASELINE config 2): LayerNorm, fused input GEMM,
+    flash attention, output GEMM.  Returns seconds per layer forward."""
+    import torch
+    eng = net.engine()
+    ses = eng.session(B, T, T, T + 8)
+    M = B * T
+    x = torch.randn(M, eng.w.d, device=eng.device)
+    pos0 = torch.zeros(B, dtype=torch.int32, device=eng.device)
+    run = lambda: eng.layer_prefill(ses, 0, x, ses.h_pf[:M], ses.act_pf[:M], T, pos0)
+    run()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        run()
+    b.record()
+    torch.cuda.synchronize()
+    eng.sessions.pop((B, T), None)
+    return a.elapsed_time(b) * 1e-3 / reps
+
+
+def cpu_baseline(net, cfg, n_layers=4, steps=8, prompt=512, L=2048):
+    """The CPU oracle (torch float32, all host threads) on a bounded sample: the first `n_layers` layers of the
+    same weights at full shape plus embedding and logits projection; 512-token prompt left-padded to 2048,
+    prefill, then `steps` greedy decode steps.  Per-step time is extrapolated linearly to 28 layers."""
+    import numpy as np
+    import torch
+    from oracle import gptj_oracle as O
+    tree = net.state["params"]
+    sub = dict(cfg, layers=n_layers)
+    keep = {}
+    for mod, leaves in tree.items():
+        if "/layer_" in mod and int(mod.split("/layer_")[1].split("/")[0]) >= n_layers:
+            continue
+        keep[mod] = {k: v.cpu() for k, v in leaves.items()}
+    model = O.Model(sub, keep, torch.float32)
+    ctx = O.left_pad(O.seeded_prompt(2, 1, prompt), L)[0]
+    t0 = time.perf_counter()
+    nxt, states = model.generate_initial(ctx, prompt)
+    t1 = time.perf_counter()
+    per = []
+    for _ in range(steps):
+        a = time.perf_counter()
+        logits, states = model.generate_once(nxt, states)
+        nxt = np.asarray([O.greedy_sample(None, logits.numpy())], np.uint32)
+        per.append(time.perf_counter() - a)
+    # cost of embedding + logits projection alone
+    x = torch.randn(1, cfg["d_model"])
+    a = time.perf_counter()
+    for _ in range(steps):
+        model.proj(x)
+    t_proj = (time.perf_counter() - a) / steps
+    t_step = float(np.median(per))
+    t_full = (t_step - t_proj) * cfg["layers"] / n_layers + t_proj
+    return {
+        "value": 1.0 / t_full, "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"CPU oracle (torch float32), {n_layers} of {cfg['layers']} layers at full shape + logits, "
+                  f"{prompt}-token prompt padded to {L}, {steps} decode steps (median {t_step * 1e3:.1f} ms/step for "
+                  f"{n_layers} layers, prefill {t1 - t0:.1f} s); per-step time extrapolated linearly to {cfg['layers']} layers",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=17)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the prefill-layer measurement")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the whole model on ONE GPU (no collectives, no sharding); "
+              f"--gpus {args.gpus} is not supported, run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from mesh_transformer import _abi, sampling
+    from mesh_transformer.transformer_shard import CausalTransformer
+    from oracle import gptj_oracle as O   # prompt generator + cpu_baseline leg only
+
+    _abi.lib()
+    dev = torch.device("cuda:0")
+    cfg = dict(CFG_6B, sampler=sampling.greedy_sample)
+    K, W = args.steps, args.warmup
+    net = CausalTransformer(cfg, synthetic_tree(cfg, 2, dev, torch.bfloat16))
+    P, L = 512, 2048
+    ctx = O.left_pad(O.seeded_prompt(2, 1, P), L)
+
+    net.generate(ctx, [P], W + K, {})                   # untimed: packs weights, allocates, records the graphs
+    timing = {"warmup": W}
+    _, out = net.generate(ctx, [P], W + K, {}, timing=timing)
+    ms_per_step = timing["decode_s"] * 1e3 / timing["decode_steps"]
+    tok_s = timing["decode_steps"] / timing["decode_s"]
+
+    ctx_mean = (P - 1) + W + (K - 1) / 2.0
+    step_bytes = decode_bytes_per_step(cfg, ctx_mean)
+    step_bw = step_bytes / (ms_per_step * 1e-3)
+
+    ses = net.engine().sessions[(1, L - 1)]
+    t_k = time_dominant_kernel(net, ses)
+    k_bytes = gemv_inproj_bytes(cfg)
+    roofline = {"bound": "hbm", "kernel": "gemv_kernel (LayerNorm + q|v|k|fc_in, N=28672, K=4096, bf16)",
+                "achieved": k_bytes / t_k / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                "frac": k_bytes / t_k / HBM_PEAK, "traffic": None, "bytes_per_launch": k_bytes,
+                "avg_launch_us": t_k * 1e6}
+
+    d, F, n = cfg["d_model"], 4 * cfg["d_model"], cfg["layers"]
+    pf_tokens = timing["prefill_tokens"]
+    pf_flops = pf_tokens * 2 * n * (4 * d * d + 2 * d * F) + n * 4 * d * pf_tokens * (pf_tokens + 1) / 2
+    prefill = {"tokens": pf_tokens, "ms": timing["prefill_s"] * 1e3, "tok_s": pf_tokens / timing["prefill_s"],
+               "tflops": pf_flops / timing["prefill_s"] / 1e12, "frac_mfma": pf_flops / timing["prefill_s"] / MFMA_BF16_PEAK}
+    if not args.no_extras:
+        Bl, Tl = 8, 2048
+        t_layer = time_prefill_layer(net, Bl, Tl)
+        Ml = Bl * Tl
+        fl = Ml * 2 * (4 * d * d + 2 * d * F) + Bl * 4 * d * Tl * (Tl + 1) / 2
+        prefill["layer_8x2048"] = {"ms": t_layer * 1e3, "tflops": fl / t_layer / 1e12, "frac_mfma": fl / t_layer / MFMA_BF16_PEAK,
+                                   "tok_s_28_layers": Ml / (t_layer * n)}
+
+    res = {
+        "metric": "GPT-J-6B bf16 decode tok/s (bs1, % HBM peak); prefill tok/s (% MFMA peak)",
+        "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE config 3: GPT-J-6B bf16 random-init N(0,0.02), batch 1, 512-token prompt "
+                               "left-padded to 2048, greedy decode; one step = one generated token",
+                   "global_batch": 1, "prompt": P, "ctx": L, "steps_per_graph": int(cfg.get("steps_per_graph", 8))},
+        "roofline": roofline,
+        "step_hbm": {"bytes": step_bytes, "achieved": step_bw / 1e9, "unit": "GB/s", "frac": step_bw / HBM_PEAK},
+        "prefill": prefill,
+    }
+    if not args.no_cpu:
+        res["cpu_baseline"] = cpu_baseline(net, cfg)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

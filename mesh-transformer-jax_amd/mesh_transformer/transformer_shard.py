@@ -4,6 +4,7 @@ on one MI355X through the HIP kernels.  Only the generate path exists here: trai
 the xmap/pjit sharding and the optimizer state are not part of this build.
 """
 import random
+import time
 
 import numpy as np
 import torch
@@ -94,7 +95,7 @@ class CausalTransformer:
 
     # ------------------------------------------------------------------ generate
     def generate(self, ctx, ctx_length, gen_length, sampler_options, return_logits=False, uniforms=None,
-                 sampler=None, return_keep_mask=False):
+                 sampler=None, return_keep_mask=False, timing=None):
         """transformer_shard.py:326-339.
 
         ctx uint32 [B, L] left-padded (device_sample.py:92-96), ctx_length [B], sampler_options a dict of
@@ -103,7 +104,9 @@ class CausalTransformer:
 
         Beyond the reference: `uniforms` float64 [B, G] in [0, 1) drive the inverse-CDF draw (default:
         drawn from an unseeded Philox stream, like the reference's unseeded key at :327);
-        `sampler` overrides config["sampler"]."""
+        `sampler` overrides config["sampler"]; `timing`, a dict with key "warmup" (decode steps left out of
+        the timed region), is filled with device-synchronised wall times: prefill_s, warmup_s, decode_s,
+        decode_steps."""
         eng = self.engine()
         self.gen_length, self.return_logits = gen_length, return_logits
         ctx = np.ascontiguousarray(np.asarray(ctx)).astype(np.int64)
@@ -152,16 +155,33 @@ class CausalTransformer:
                     raise ValueError(f"uniforms must have shape {(B, G)}")
                 ses.uniforms[:, :G].copy_(torch.from_numpy(np.ascontiguousarray(u)))
             # --- prefill
+            rect = None
             if Tp > 0:
                 rect = torch.from_numpy(np.ascontiguousarray(ctx[:, Lc - 1 - Tp:Lc - 1]).astype(np.int32)).to(dev)
-                eng.prefill(ses, rect, Tp)
-            # --- decode
             logits_out = torch.empty(B, G, eng.w.V, dtype=torch.float32, device=dev) if return_logits else None
             masks = torch.empty(G, B, eng.w.V, dtype=torch.uint8, device=dev) if return_keep_mask else None   # [step, row, V]
+
+            def clock():
+                torch.cuda.synchronize(dev)
+                return time.perf_counter()
+
+            t0 = clock() if timing is not None else 0.0
+            if Tp > 0:
+                eng.prefill(ses, rect, Tp)
+            t1 = clock() if timing is not None else 0.0
+            # --- decode
             if kind is None:
                 self._decode_host_sampler(eng, ses, G, sampler, opts, logits_out)
+            elif timing is None:
+                self._decode(eng, ses, 0, G, kind, logits_out, masks)
             else:
-                self._decode(eng, ses, G, kind, logits_out, masks)
+                W = min(int(timing.get("warmup", 0)), G - 1)
+                self._decode(eng, ses, 0, W, kind, logits_out, masks)
+                t2 = clock()
+                self._decode(eng, ses, W, G, kind, logits_out, masks)
+                t3 = clock()
+                timing.update(prefill_s=t1 - t0, prefill_tokens=B * Tp, warmup_s=t2 - t1, decode_s=t3 - t2,
+                              decode_steps=G - W)
             torch.cuda.synchronize(dev)
             toks = ses.out_tokens[:, :G].cpu().numpy().astype(np.uint32)[:, :, None]
             final_state = (toks[:, -1], ses, None)
@@ -192,10 +212,10 @@ class CausalTransformer:
             eng.sample_nucleus(ses, ses.out_tokens, ses.top_p, ses.temp, ses.top_k if ses.use_top_k else None,
                                ses.uniforms, keep_mask=keep_mask)
 
-    def _decode(self, eng, ses, G, kind, logits_out, masks):
+    def _decode(self, eng, ses, t, G, kind, logits_out, masks):
+        """Decode steps t .. G-1."""
         spg = int(self.config.get("steps_per_graph", 8))
         eager = spg <= 0 or logits_out is not None or masks is not None
-        t = 0
         while t < G:
             if eager or t == 0:
                 # the first step always runs eagerly: it also performs the kernels' one-time setup

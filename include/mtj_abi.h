@@ -118,16 +118,29 @@ int mtj_attn_prefill(const void* q, const void* k_cache, const void* v_t, const 
 
 /* One-token attention over the K/V window (decode_once, layers.py:316-344): for sequence b the valid
  * slots are [0, min(pos[b]+1, Tcap)).  q float32 [B,H,dh]; caches in `dtype`; out [B, ld_out] in out_dtype
- * (columns h*dh + c).  `work` needs mtj_attn_decode_work_bytes(B, H, dh, Tcap) bytes. */
+ * (columns h*dh + c).  `work` (16-byte aligned, mtj_attn_decode_work_bytes(B, H, dh, Tcap) bytes) holds the per-split
+ * partial results between the two launches this call makes; calls sharing one `work` must not overlap. */
 int64_t mtj_attn_decode_work_bytes(int64_t B, int64_t H, int64_t dh, int64_t Tcap);
 int mtj_attn_decode(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,
                     int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
                     void* work, void* stream);
 
+/* Next-step embedding fused into the samplers: when `w` is non-NULL the sampler also writes
+ * x_next[b, :] = w[token, :] + bias (EmbeddingShard of the token it just chose, layers.py:187-202), which is the
+ * input of the next decode step (transformer_shard.py:107). */
+typedef struct {
+  const void* w;      /* [n_vocab, d] in dtype, or NULL */
+  const float* bias;  /* [d] */
+  float* x_next;      /* [B, d] */
+  int64_t d;
+  int32_t dtype;
+} mtj_next_embed;
+
 /* Greedy sampler through the reference's sampler contract (transformer_shard.py:203): lowest index among
  * maxima.  Writes tok[b], out_tokens[b * ld_tokens + (pos[b] - pos_start[b])], then pos[b] += 1. */
 int mtj_sample_greedy(const float* logits, int64_t B, int64_t V, int32_t* tok, int32_t* out_tokens,
-                      int64_t ld_tokens, int32_t* pos, const int32_t* pos_start, void* stream);
+                      int64_t ld_tokens, int32_t* pos, const int32_t* pos_start, const mtj_next_embed* next,
+                      void* stream);
 
 /* nucleaus_sample (sampling.py:10-44) with the Gumbel draw replaced by an inverse-CDF draw from
  * host-supplied uniforms: filter on the RAW logits (optional top_k, then top_p, float64 softmax and
@@ -140,7 +153,7 @@ int64_t mtj_sample_work_bytes(int64_t B, int64_t V);
 int mtj_sample_nucleus(const float* logits, int64_t B, int64_t V, const double* top_p, const double* temp,
                        const int32_t* top_k, const double* uniforms, int64_t ld_u, int32_t* tok,
                        int32_t* out_tokens, int64_t ld_tokens, int32_t* pos, const int32_t* pos_start,
-                       uint8_t* keep_mask, float* filtered, void* work, void* stream);
+                       uint8_t* keep_mask, float* filtered, void* work, const mtj_next_embed* next, void* stream);
 
 #ifdef __cplusplus
 }

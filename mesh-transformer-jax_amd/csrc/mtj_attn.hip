@@ -203,129 +203,147 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__
 }
 
 // ------------------------------------------------------------------------------------------------
-// Decode.  Grid (splits, H, B); each workgroup reduces a contiguous range of window slots to a partial
-// (max, sum, weighted V) that attn_combine_kernel merges.  16-byte loads: LPK lanes cover one key row.
+// Decode.  Grid (splits, H, B); each workgroup reduces 64 window slots to a partial (max, sum, weighted V)
+// and attn_combine_kernel merges the non-empty partials of a (sequence, head).  (Merging in the same launch,
+// by the last workgroup to arrive, needs a device-scope fence per workgroup; on this multi-die GPU that
+// fence writes back the L2 and made the kernel 6x slower than the two launches.)  16-byte loads: LPK lanes
+// cover one key row; all K and V loads of a workgroup are requested up front (V does not depend on the
+// scores).
+constexpr int DEC_CHUNK = 64;
+
 template <typename T, int DH>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const T* __restrict__ kc,
                                                           const T* __restrict__ vc, const int32_t* __restrict__ pos,
-                                                          int H, int Tcap, int chunk, float* __restrict__ work) {
+                                                          int H, int Tcap, float* __restrict__ work) {
   constexpr int EPC = 16 / sizeof(T);
   constexpr int LPK = DH / EPC;      // lanes per key row
   constexpr int KPL = 64 / LPK;      // keys per wavefront load
-  static_assert(LPK <= 64 && 64 % LPK == 0, "head dim does not map onto a wavefront");
-  extern __shared__ __align__(16) float sm[];   // [chunk] scores, then [4][DH] partial outputs
-  __shared__ float red[8];
+  constexpr int NI = DEC_CHUNK / (4 * KPL);   // loads per lane for K (and for V)
+  static_assert(LPK <= 64 && 64 % LPK == 0 && NI >= 1, "head dim does not map onto a wavefront");
+  __shared__ float sc[DEC_CHUNK];
+  __shared__ float part[4][DH];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z, S = gridDim.x;
   const int64_t bh = (int64_t)b * H + h;
   const int nvalid = (pos[b] + 1 < Tcap) ? pos[b] + 1 : Tcap;
-  const int k0 = split * chunk;
-  const int k1 = (k0 + chunk < nvalid) ? k0 + chunk : nvalid;
+  const int k0 = split * DEC_CHUNK;
+  const int nk = (k0 + DEC_CHUNK < nvalid) ? DEC_CHUNK : nvalid - k0;     // <= 0: nothing in this range
   float* wout = work + (bh * S + split) * (DH + 2);
-  if (k1 <= k0) {  // empty range
-    for (int e = tid; e < DH; e += 256) wout[2 + e] = 0.f;
-    if (tid == 0) { wout[0] = -INFINITY; wout[1] = 0.f; }
-    return;
-  }
-  const int nk = k1 - k0;
   const int sub = lane / LPK, el = (lane % LPK) * EPC;
-  float qv[EPC];
-#pragma unroll
-  for (int j = 0; j < EPC; ++j) qv[j] = q[bh * DH + el + j];
-  const float scale = rsqrtf((float)DH);
 
-  // ---- scores
-  const T* kbase = kc + (bh * Tcap + k0) * DH;
-  for (int kk = wave * KPL + sub; kk < nk + KPL; kk += 4 * KPL) {   // uniform trip count per wavefront
-    float d = 0.f;
-    if (kk < nk) {
-      const uint32x4 w = *reinterpret_cast<const uint32x4*>(kbase + (int64_t)kk * DH + el);
-      if (sizeof(T) == 2) {
-        d = bf16_lo(w.x) * qv[0] + bf16_hi(w.x) * qv[1 % EPC] + bf16_lo(w.y) * qv[2 % EPC] + bf16_hi(w.y) * qv[3 % EPC] +
-            bf16_lo(w.z) * qv[4 % EPC] + bf16_hi(w.z) * qv[5 % EPC] + bf16_lo(w.w) * qv[6 % EPC] + bf16_hi(w.w) * qv[7 % EPC];
-      } else {
-        d = __uint_as_float(w.x) * qv[0] + __uint_as_float(w.y) * qv[1] + __uint_as_float(w.z) * qv[2] +
-            __uint_as_float(w.w) * qv[3];
+  if (nk > 0) {
+    // ---- request every K and V row of the range
+    uint32x4 kr[NI], vr[NI];
+    const T* kbase = kc + (bh * Tcap + k0) * DH + el;
+    const T* vbase = vc + (bh * Tcap + k0) * DH + el;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int kk = (i * 4 + wave) * KPL + sub;
+      if (kk < nk) {
+        kr[i] = *reinterpret_cast<const uint32x4*>(kbase + (int64_t)kk * DH);
+        vr[i] = *reinterpret_cast<const uint32x4*>(vbase + (int64_t)kk * DH);
+      }
+    }
+    float qv[EPC];
+#pragma unroll
+    for (int j = 0; j < EPC; ++j) qv[j] = q[bh * DH + el + j];
+    const float scale = rsqrtf((float)DH);
+    // ---- scores
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int kk = (i * 4 + wave) * KPL + sub;
+      float d = 0.f;
+      if (kk < nk) {
+        const uint32x4 w = kr[i];
+        if (sizeof(T) == 2) {
+          d = bf16_lo(w.x) * qv[0] + bf16_hi(w.x) * qv[1 % EPC] + bf16_lo(w.y) * qv[2 % EPC] + bf16_hi(w.y) * qv[3 % EPC] +
+              bf16_lo(w.z) * qv[4 % EPC] + bf16_hi(w.z) * qv[5 % EPC] + bf16_lo(w.w) * qv[6 % EPC] + bf16_hi(w.w) * qv[7 % EPC];
+        } else {
+          d = __uint_as_float(w.x) * qv[0] + __uint_as_float(w.y) * qv[1] + __uint_as_float(w.z) * qv[2] +
+              __uint_as_float(w.w) * qv[3];
+        }
+      }
+#pragma unroll
+      for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o);
+      if (kk < nk && (lane % LPK) == 0) sc[kk] = d * scale;
+    }
+    __syncthreads();
+    // ---- softmax statistics of the range (64 scores: one wavefront's worth, every wavefront redoes it)
+    const float sv = (lane < nk) ? sc[lane] : -INFINITY;
+    const float m = wave_max(sv);
+    const float pv = (lane < nk) ? expf(sv - m) : 0.f;
+    const float l = wave_sum(pv);
+    // ---- weighted V from the registers
+    float acc[EPC];
+#pragma unroll
+    for (int j = 0; j < EPC; ++j) acc[j] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int kk = (i * 4 + wave) * KPL + sub;
+      const float p = __shfl(pv, kk < nk ? kk : 0);
+      if (kk < nk) {
+        const uint32x4 w = vr[i];
+        if (sizeof(T) == 2) {
+          acc[0] += p * bf16_lo(w.x); acc[1 % EPC] += p * bf16_hi(w.x);
+          acc[2 % EPC] += p * bf16_lo(w.y); acc[3 % EPC] += p * bf16_hi(w.y);
+          acc[4 % EPC] += p * bf16_lo(w.z); acc[5 % EPC] += p * bf16_hi(w.z);
+          acc[6 % EPC] += p * bf16_lo(w.w); acc[7 % EPC] += p * bf16_hi(w.w);
+        } else {
+          acc[0] += p * __uint_as_float(w.x); acc[1] += p * __uint_as_float(w.y);
+          acc[2] += p * __uint_as_float(w.z); acc[3] += p * __uint_as_float(w.w);
+        }
       }
     }
 #pragma unroll
-    for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o);
-    if (kk < nk && (lane % LPK) == 0) sm[kk] = d * scale;
+    for (int j = 0; j < EPC; ++j)
+#pragma unroll
+      for (int o = 32; o >= LPK; o >>= 1) acc[j] += __shfl_xor(acc[j], o);
+    if (lane < LPK)
+#pragma unroll
+      for (int j = 0; j < EPC; ++j) part[wave][el + j] = acc[j];
+    __syncthreads();
+    for (int e = tid; e < DH; e += 256) wout[2 + e] = (part[0][e] + part[1][e]) + (part[2][e] + part[3][e]);
+    if (tid == 0) { wout[0] = m; wout[1] = l; }
   }
-  __syncthreads();
-  // ---- softmax statistics of the range
-  float m = -INFINITY;
-  for (int i = tid; i < nk; i += 256) m = fmaxf(m, sm[i]);
-  m = wave_max(m);
-  if (lane == 0) red[wave] = m;
-  __syncthreads();
-  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-  float l = 0.f;
-  for (int i = tid; i < nk; i += 256) {
-    const float p = expf(sm[i] - m);
-    sm[i] = p;
-    l += p;
-  }
-  l = wave_sum(l);
-  if (lane == 0) red[4 + wave] = l;
-  __syncthreads();
-  l = (red[4] + red[5]) + (red[6] + red[7]);
 
-  // ---- weighted V
-  float acc[EPC];
-#pragma unroll
-  for (int j = 0; j < EPC; ++j) acc[j] = 0.f;
-  const T* vbase = vc + (bh * Tcap + k0) * DH;
-  for (int kk = wave * KPL + sub; kk < nk; kk += 4 * KPL) {
-    const uint32x4 w = *reinterpret_cast<const uint32x4*>(vbase + (int64_t)kk * DH + el);
-    const float p = sm[kk];
-    if (sizeof(T) == 2) {
-      acc[0] += p * bf16_lo(w.x); acc[1 % EPC] += p * bf16_hi(w.x);
-      acc[2 % EPC] += p * bf16_lo(w.y); acc[3 % EPC] += p * bf16_hi(w.y);
-      acc[4 % EPC] += p * bf16_lo(w.z); acc[5 % EPC] += p * bf16_hi(w.z);
-      acc[6 % EPC] += p * bf16_lo(w.w); acc[7 % EPC] += p * bf16_hi(w.w);
-    } else {
-      acc[0] += p * __uint_as_float(w.x); acc[1] += p * __uint_as_float(w.y);
-      acc[2] += p * __uint_as_float(w.z); acc[3] += p * __uint_as_float(w.w);
-    }
-  }
-#pragma unroll
-  for (int j = 0; j < EPC; ++j)
-#pragma unroll
-    for (int o = 32; o >= LPK; o >>= 1) acc[j] += __shfl_xor(acc[j], o);
-  __syncthreads();                       // scores no longer needed: reuse sm as [4][DH]
-  if (lane < LPK)
-#pragma unroll
-    for (int j = 0; j < EPC; ++j) sm[wave * DH + el + j] = acc[j];
-  __syncthreads();
-  for (int e = tid; e < DH; e += 256) wout[2 + e] = (sm[e] + sm[DH + e]) + (sm[2 * DH + e] + sm[3 * DH + e]);
-  if (tid == 0) { wout[0] = m; wout[1] = l; }
 }
 
+// Grid (H, B): merge the partials of the non-empty splits.
 template <int DH>
-__global__ void attn_combine_kernel(const float* __restrict__ work, int S, int H, void* __restrict__ out,
-                                    int64_t ld_out, int out_dtype) {
-  const int h = blockIdx.x, b = blockIdx.y, e = threadIdx.x;
-  const float* w = work + ((int64_t)b * H + h) * S * (DH + 2);
-  float m = -INFINITY;
-  for (int s = 0; s < S; ++s) m = fmaxf(m, w[s * (DH + 2)]);
-  float l = 0.f, acc = 0.f;
-  for (int s = 0; s < S; ++s) {
-    const float f = expf(w[s * (DH + 2)] - m);
-    l += f * w[s * (DH + 2) + 1];
-    acc += f * w[s * (DH + 2) + 2 + e];
+__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ work, const int32_t* __restrict__ pos,
+                                                           int S, int H, int Tcap, void* __restrict__ out, int64_t ld_out,
+                                                           int out_dtype) {
+  __shared__ float wgt[64];
+  const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int64_t bh = (int64_t)b * H + h;
+  const int nvalid = (pos[b] + 1 < Tcap) ? pos[b] + 1 : Tcap;
+  const int ns = (nvalid + DEC_CHUNK - 1) / DEC_CHUNK;    // non-empty splits (<= S <= 64)
+  const float* wb = work + bh * S * (DH + 2);
+  if (tid < 64) {
+    const float ms = (tid < ns) ? wb[(int64_t)tid * (DH + 2)] : -INFINITY;
+    const float ls = (tid < ns) ? wb[(int64_t)tid * (DH + 2) + 1] : 0.f;
+    const float mm = wave_max(ms);
+    const float f = (tid < ns) ? expf(ms - mm) : 0.f;
+    const float lt = wave_sum(f * ls);
+    wgt[tid] = f / lt;
   }
-  store_as(out, (int64_t)b * ld_out + h * DH + e, acc / l, out_dtype);
+  __syncthreads();
+  for (int e = tid; e < DH; e += 256) {
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int s2 = 0;
+    for (; s2 + 3 < ns; s2 += 4) {
+      a0 += wgt[s2] * wb[(int64_t)s2 * (DH + 2) + 2 + e];
+      a1 += wgt[s2 + 1] * wb[(int64_t)(s2 + 1) * (DH + 2) + 2 + e];
+      a2 += wgt[s2 + 2] * wb[(int64_t)(s2 + 2) * (DH + 2) + 2 + e];
+      a3 += wgt[s2 + 3] * wb[(int64_t)(s2 + 3) * (DH + 2) + 2 + e];
+    }
+    for (; s2 < ns; ++s2) a0 += wgt[s2] * wb[(int64_t)s2 * (DH + 2) + 2 + e];
+    store_as(out, (int64_t)b * ld_out + h * DH + e, (a0 + a1) + (a2 + a3), out_dtype);
+  }
 }
 
-int decode_splits(int64_t B, int64_t H, int64_t Tcap) {
-  int64_t s = (1024 + B * H - 1) / (B * H);
-  const int64_t smax = (Tcap + 63) / 64;
-  if (s > smax) s = smax;
-  if (s < 1) s = 1;
-  return (int)s;
-}
+int decode_splits(int64_t Tcap) { return (int)((Tcap + DEC_CHUNK - 1) / DEC_CHUNK); }
 
 }  // namespace
 
@@ -356,7 +374,7 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
 }
 
 extern "C" int64_t mtj_attn_decode_work_bytes(int64_t B, int64_t H, int64_t dh, int64_t Tcap) {
-  return B * H * (int64_t)decode_splits(B, H, Tcap) * (dh + 2) * (int64_t)sizeof(float);
+  return B * H * (int64_t)decode_splits(Tcap) * (dh + 2) * (int64_t)sizeof(float);
 }
 
 extern "C" int mtj_attn_decode(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,
@@ -366,20 +384,19 @@ extern "C" int mtj_attn_decode(const float* q, const void* k_cache, const void* 
   MTJ_REQUIRE(B > 0 && H > 0 && Tcap > 0 && ld_out >= H * dh && B < 65536 && H < 65536, MTJ_EINVAL,
               "mtj_attn_decode: bad shape");
   MTJ_REQUIRE(out_dtype == MTJ_F32 || out_dtype == MTJ_BF16, MTJ_EDTYPE, "mtj_attn_decode: out_dtype %d", out_dtype);
-  MTJ_REQUIRE(mtj_aligned16(q) && mtj_aligned16(k_cache) && mtj_aligned16(v_cache), MTJ_EALIGN,
+  MTJ_REQUIRE(mtj_aligned16(q) && mtj_aligned16(k_cache) && mtj_aligned16(v_cache) && mtj_aligned16(work), MTJ_EALIGN,
               "mtj_attn_decode: pointers must be 16-byte aligned");
-  const int S = decode_splits(B, H, Tcap);
-  const int chunk = (int)((Tcap + S - 1) / S);
-  const size_t lds = sizeof(float) * (size_t)(chunk > 4 * dh ? chunk : 4 * dh);
-  MTJ_REQUIRE(lds <= 60 * 1024, MTJ_ELIMIT, "mtj_attn_decode: window chunk %d too large", chunk);
+  const int S = decode_splits(Tcap);
+  MTJ_REQUIRE(S <= 64, MTJ_ELIMIT, "mtj_attn_decode: window of %lld slots exceeds %d", (long long)Tcap, 64 * DEC_CHUNK);
+  float* partials = reinterpret_cast<float*>(work);
   dim3 grid((unsigned)S, (unsigned)H, (unsigned)B);
   hipStream_t s = (hipStream_t)stream;
-#define MTJ_DECODE(T, DH)                                                                                       \
-  do {                                                                                                          \
-    attn_decode_kernel<T, DH><<<grid, 256, lds, s>>>(q, (const T*)k_cache, (const T*)v_cache, pos, (int)H,      \
-                                                     (int)Tcap, chunk, (float*)work);                           \
-    attn_combine_kernel<DH><<<dim3((unsigned)H, (unsigned)B), DH, 0, s>>>((const float*)work, S, (int)H, out,   \
-                                                                          ld_out, out_dtype);                   \
+#define MTJ_DECODE(T, DH)                                                                                         \
+  do {                                                                                                            \
+    attn_decode_kernel<T, DH><<<grid, 256, 0, s>>>(q, (const T*)k_cache, (const T*)v_cache, pos, (int)H, (int)Tcap, \
+                                                   partials);                                                     \
+    attn_combine_kernel<DH><<<dim3((unsigned)H, (unsigned)B), 256, 0, s>>>(partials, pos, S, (int)H, (int)Tcap, out, \
+                                                                           ld_out, out_dtype);                    \
   } while (0)
   if (dtype == MTJ_BF16 && dh == 256) MTJ_DECODE(bf16_t, 256);
   else if (dtype == MTJ_BF16 && dh == 64) MTJ_DECODE(bf16_t, 64);

@@ -83,41 +83,72 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 }
 
 // ---------------------------------------------------------------- fused input-projection epilogue
-// One output element (row m, column n) of q|v|k|fc_in.  `own` is the accumulator of column n,
-// `partner` the accumulator of column n ^ 1 of the same row (needed by the interleaved rotation,
-// layers.py:137-148: out[2i] = x[2i] cos - x[2i+1] sin, out[2i+1] = x[2i+1] cos + x[2i] sin).
-__device__ __forceinline__ void inproj_store(const mtj_inproj& ip, const float* __restrict__ b1, int kv_dtype,
-                                             int64_t m, int64_t n, float own, float partner) {
+// One output element (row m, column n) of q|v|k|fc_in, in two halves so that a bandwidth-bound caller can
+// issue the loads (position, sin/cos, bias) long before the accumulator is ready: inproj_prepare does every
+// global read, inproj_finish only arithmetic and stores.  `own` is the accumulator of column n, `partner`
+// that of column n ^ 1 of the same row (the interleaved rotation of layers.py:137-148:
+// out[2i] = x[2i] cos - x[2i+1] sin, out[2i+1] = x[2i+1] cos + x[2i] sin).
+struct inproj_pre {
+  int kind;        // 0 q, 1 v, 2 k, 3 fc_in, -1 nothing to store (padding row)
+  float sn, cs;    // rotation of this element (cs = 1, sn = 0 outside the rotary dims)
+  float bias;      // fc_in bias
+  int64_t idx;     // destination element in q / k_cache / v_cache / act
+  int64_t idx_t;   // destination in v_t, or -1
+};
+
+__device__ __forceinline__ inproj_pre inproj_prepare(const mtj_inproj& ip, const float* __restrict__ b1, int64_t m,
+                                                     int64_t n) {
+  inproj_pre p;
+  p.sn = 0.f; p.cs = 1.f; p.bias = 0.f; p.idx = 0; p.idx_t = -1;
   const int d = ip.n_heads * ip.d_head;
   const int b = (int)(m / ip.Tp), t = (int)(m - (int64_t)b * ip.Tp);
-  const int pos = ip.pos0[b] + t;
   if (n >= 3 * (int64_t)d) {  // fc_in -> gelu
     const int64_t c = n - 3 * (int64_t)d;
-    const float g = gelu_tanh(own + b1[c]);
-    store_as(ip.act, m * ip.ld_act + d + c, g, ip.act_dtype);
-    return;
+    p.kind = 3;
+    p.bias = b1[c];
+    p.idx = m * ip.ld_act + d + c;
+    return p;
   }
-  if (pos < 0) return;  // left padding: nothing reaches the cache
-  const int seg = (int)(n / d);          // 0 q, 1 v, 2 k
+  const int pos = ip.pos0[b] + t;
+  if (pos < 0) { p.kind = -1; return p; }  // left padding: nothing reaches the cache
+  const int seg = (int)(n / d);            // 0 q, 1 v, 2 k
   const int c = (int)(n - (int64_t)seg * d);
   const int h = c / ip.d_head, e = c - h * ip.d_head;
-  float val = own;
+  p.kind = seg;
   if (seg != 1 && e < ip.rotary_dims) {
-    const int p = pos < ip.max_pos ? pos : ip.max_pos - 1;
-    const float sn = ip.sin_tab[(int64_t)p * (ip.rotary_dims / 2) + (e >> 1)];
-    const float cs = ip.cos_tab[(int64_t)p * (ip.rotary_dims / 2) + (e >> 1)];
-    val = (e & 1) ? (own * cs + partner * sn) : (own * cs - partner * sn);
+    const int pp = pos < ip.max_pos ? pos : ip.max_pos - 1;
+    const float sn = ip.sin_tab[(int64_t)pp * (ip.rotary_dims / 2) + (e >> 1)];
+    p.cs = ip.cos_tab[(int64_t)pp * (ip.rotary_dims / 2) + (e >> 1)];
+    p.sn = (e & 1) ? sn : -sn;
   }
   if (seg == 0) {
-    const int64_t idx = (((int64_t)b * ip.n_heads + h) * ip.Tp + t) * ip.d_head + e;
-    store_as(ip.q, idx, val, ip.q_dtype);
+    p.idx = (((int64_t)b * ip.n_heads + h) * ip.Tp + t) * ip.d_head + e;
   } else {
     const int slot = pos % ip.Tcap;
-    const int64_t idx = (((int64_t)b * ip.n_heads + h) * ip.Tcap + slot) * ip.d_head + e;
-    store_as(seg == 1 ? ip.v_cache : ip.k_cache, idx, val, kv_dtype);
-    if (seg == 1 && ip.v_t && pos < ip.ldvt) {  // transposed copy, indexed by position like the cache
-      const int64_t it = (((int64_t)b * ip.n_heads + h) * ip.d_head + e) * ip.ldvt + pos;
-      store_as(ip.v_t, it, val, kv_dtype);
-    }
+    p.idx = (((int64_t)b * ip.n_heads + h) * ip.Tcap + slot) * ip.d_head + e;
+    if (seg == 1 && ip.v_t && pos < ip.ldvt)   // transposed copy, indexed by position like the cache
+      p.idx_t = (((int64_t)b * ip.n_heads + h) * ip.d_head + e) * ip.ldvt + pos;
   }
+  return p;
+}
+
+__device__ __forceinline__ void inproj_finish(const mtj_inproj& ip, int kv_dtype, const inproj_pre& p, float own,
+                                              float partner) {
+  if (p.kind < 0) return;
+  if (p.kind == 3) {
+    store_as(ip.act, p.idx, gelu_tanh(own + p.bias), ip.act_dtype);
+    return;
+  }
+  const float val = own * p.cs + partner * p.sn;
+  if (p.kind == 0) {
+    store_as(ip.q, p.idx, val, ip.q_dtype);
+  } else {
+    store_as(p.kind == 1 ? ip.v_cache : ip.k_cache, p.idx, val, kv_dtype);
+    if (p.idx_t >= 0) store_as(ip.v_t, p.idx_t, val, kv_dtype);
+  }
+}
+
+__device__ __forceinline__ void inproj_store(const mtj_inproj& ip, const float* __restrict__ b1, int kv_dtype,
+                                             int64_t m, int64_t n, float own, float partner) {
+  inproj_finish(ip, kv_dtype, inproj_prepare(ip, b1, m, n), own, partner);
 }

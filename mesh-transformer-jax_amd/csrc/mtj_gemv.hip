@@ -46,137 +46,164 @@ struct gemv_args {
   mtj_inproj ip;
 };
 
-// R rows per wavefront, U 16-byte loads in flight per row.
-template <typename T, int R, int U>
+// One workgroup of 16 wavefronts per CU, all resident at once (a second round of workgroups would pay the
+// prologue and the drain of the memory pipeline twice).  The rows (row pairs for the fused input projection,
+// whose rotary epilogue needs both halves of a pair) are dealt out in equal contiguous ranges over all
+// wavefronts of the grid.  Nothing on the streaming path depends on a second global load: x is requested
+// first, then the first U KiB of weights (so the LayerNorm prologue overlaps the first HBM round trip), and
+// every epilogue operand (position, sin/cos, biases, the residual) is fetched up front by the lane that
+// will finish that row - under load a dependent load costs tens of microseconds.
+template <typename T, int U>
 __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   extern __shared__ __align__(16) float xs[];
   __shared__ float red[2][16];
   constexpr int EPC = chunk<T>::EPC;
+  constexpr int STEP = 64 * EPC;  // elements one wavefront covers per load
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
   const int K = (int)a.K;
+  const T* __restrict__ W = reinterpret_cast<const T*>(a.W);
+
+  const bool pairs = a.epi == MTJ_EPI_INPROJ;
+  const int64_t upw = pairs ? 2 : 1;
+  const int64_t units = a.N / upw;
+  const int64_t gw = (int64_t)blockIdx.x * nwaves + wave, nw_total = (int64_t)gridDim.x * nwaves;
+  const int64_t row0 = (units * gw / nw_total) * upw, row1 = (units * (gw + 1) / nw_total) * upw;
+  const int nrows = (int)(row1 - row0);                     // <= 64 (the host sizes the grid for that)
+
+  // ---- x first (4 values per thread while K <= 4096; the general loop below covers the rest) ...
+  const bool ln = a.ln_scale != nullptr;
+  floatx4 xv = {0.f, 0.f, 0.f, 0.f};
+  const bool fast_x = ln && K == 4 * (int)blockDim.x;
+  if (fast_x) xv = *reinterpret_cast<const floatx4*>(a.x + 4 * tid);
+  // ---- ... then the epilogue operands of "my" row (lane j finishes row row0 + j) ...
+  inproj_pre pre;
+  pre.kind = -1;
+  float pre_add = 0.f;
+  if (lane < nrows) {
+    const int64_t n = row0 + lane;
+    if (pairs) pre = inproj_prepare(a.ip, a.bias, 0, n);
+    else {
+      pre_add = a.bias ? a.bias[n] : 0.f;
+      if (a.epi == MTJ_EPI_RESID) pre_add += reinterpret_cast<const float*>(a.out)[n];
+    }
+  }
+  // ---- ... then the first tile of weights
+  uint32x4 w[U];
+  if (nrows > 0) {
+    const T* rowp = W + row0 * a.K;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = u * STEP + lane * EPC;
+      if (k < K) w[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(rowp + k));
+    }
+  }
 
   // ---- stage x (with LayerNorm if asked) into LDS
-  if (a.ln_scale) {
+  if (ln) {
     float s = 0.f;
-    for (int k = tid; k < K; k += blockDim.x) {
-      const float v = a.x[k];
-      xs[k] = v;
-      s += v;
+    if (fast_x) {
+      s = (xv.x + xv.y) + (xv.z + xv.w);
+    } else {
+      for (int k = tid; k < K; k += blockDim.x) {
+        const float v = a.x[k];
+        xs[k] = v;
+        s += v;
+      }
     }
     s = wave_sum(s);
     if (lane == 0) red[0][wave] = s;
     __syncthreads();
     float tot = 0.f;
-    for (int w = 0; w < nwaves; ++w) tot += red[0][w];
+    for (int i = 0; i < nwaves; ++i) tot += red[0][i];
     const float mean = tot / (float)K;
     float q = 0.f;
-    for (int k = tid; k < K; k += blockDim.x) {
-      const float t = xs[k] - mean;
-      q += t * t;
+    if (fast_x) {
+      const floatx4 t = xv - mean;
+      q = (t.x * t.x + t.y * t.y) + (t.z * t.z + t.w * t.w);
+    } else {
+      for (int k = tid; k < K; k += blockDim.x) {
+        const float t = xs[k] - mean;
+        q += t * t;
+      }
     }
     q = wave_sum(q);
     if (lane == 0) red[1][wave] = q;
     __syncthreads();
     float var = 0.f;
-    for (int w = 0; w < nwaves; ++w) var += red[1][w];
+    for (int i = 0; i < nwaves; ++i) var += red[1][i];
     const float inv = rsqrtf(var / (float)K + 1e-5f);
-    for (int k = tid; k < K; k += blockDim.x)
-      xs[k] = (a.ln_scale[k] * inv) * (xs[k] - mean) + a.ln_offset[k];
+    if (fast_x) {
+      const floatx4 sc = *reinterpret_cast<const floatx4*>(a.ln_scale + 4 * tid);
+      const floatx4 of = *reinterpret_cast<const floatx4*>(a.ln_offset + 4 * tid);
+      *reinterpret_cast<floatx4*>(xs + 4 * tid) = (sc * inv) * (xv - mean) + of;
+    } else {
+      for (int k = tid; k < K; k += blockDim.x)
+        xs[k] = (a.ln_scale[k] * inv) * (xs[k] - mean) + a.ln_offset[k];
+    }
   } else {
     for (int k = tid * 4; k < K; k += blockDim.x * 4)
       *reinterpret_cast<floatx4*>(xs + k) = *reinterpret_cast<const floatx4*>(a.x + k);
   }
   __syncthreads();
 
-  // ---- stream the rows of this wavefront
-  const int64_t n0 = ((int64_t)blockIdx.x * nwaves + wave) * R;
-  if (n0 >= a.N) return;
-  const T* __restrict__ W = reinterpret_cast<const T*>(a.W);
-  const T* rows[R];
+  // ---- stream my rows; lane r keeps the sum of row r
+  const int tpr = (K + STEP * U - 1) / (STEP * U);          // tiles per row
+  float mine = 0.f;
+  for (int r = 0; r < nrows; ++r) {
+    const T* rowp = W + (row0 + r) * a.K;
+    float acc = 0.f;
+    for (int kt = 0; kt < tpr; ++kt) {
+      if (r | kt) {   // tile (0, 0) is already in registers
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int64_t n = (n0 + r < a.N) ? n0 + r : a.N - 1;  // clamp: duplicates are never stored
-    rows[r] = W + n * a.K;
-  }
-  float acc[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) acc[r] = 0.f;
-
-  const int step = 64 * EPC;            // elements one wavefront covers per load
-  const int kfull = (K / (step * U)) * (step * U);
-  int k = lane * EPC;
-  for (; k < kfull; k += step * U) {
-    uint32x4 w[U][R];
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int r = 0; r < R; ++r)
-        w[u][r] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(rows[r] + k + u * step));
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int r = 0; r < R; ++r) chunk<T>::fma(w[u][r], xs + k + u * step, acc[r]);
-  }
-  for (; k < K; k += step) {
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const uint32x4 w = *reinterpret_cast<const uint32x4*>(rows[r] + k);
-      chunk<T>::fma(w, xs + k, acc[r]);
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
-
-  // ---- epilogue: lane r finishes row n0 + r
-  if (lane < R) {
-    float own = acc[0], partner = acc[0];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-      if (lane == r) {
-        own = acc[r];
-        partner = acc[(r ^ 1) < R ? (r ^ 1) : r];
+        for (int u = 0; u < U; ++u) {
+          const int k = (kt * U + u) * STEP + lane * EPC;
+          if (k < K) w[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(rowp + k));
+        }
       }
-    const int64_t n = n0 + lane;
-    if (n < a.N) {
-      if (a.epi == MTJ_EPI_STORE) {
-        store_as(a.out, n, own + (a.bias ? a.bias[n] : 0.f), a.out_dtype);
-      } else if (a.epi == MTJ_EPI_RESID) {
-        float* o = reinterpret_cast<float*>(a.out);
-        o[n] += own + (a.bias ? a.bias[n] : 0.f);
-      } else {
-        inproj_store(a.ip, a.bias, a.kv_dtype, 0, n, own, partner);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int k = (kt * U + u) * STEP + lane * EPC;
+        if (k < K) chunk<T>::fma(w[u], xs + k, acc);
       }
     }
+    const float sum = wave_sum(acc);
+    if (lane == r) mine = sum;
+  }
+
+  // ---- epilogue: every lane finishes its own row
+  if (pairs) {
+    const float partner = __shfl_xor(mine, 1);
+    if (lane < nrows) inproj_finish(a.ip, a.kv_dtype, pre, mine, partner);
+  } else if (lane < nrows) {
+    const int64_t n = row0 + lane;
+    if (a.epi == MTJ_EPI_STORE) store_as(a.out, n, mine + pre_add, a.out_dtype);
+    else reinterpret_cast<float*>(a.out)[n] = mine + pre_add;
   }
 }
 
-template <typename T, int R, int U>
-int launch(const gemv_args& a, int waves, hipStream_t s) {
-  const int64_t rows_per_block = (int64_t)waves * R;
-  const unsigned grid = (unsigned)((a.N + rows_per_block - 1) / rows_per_block);
+template <typename T, int U>
+int launch(const gemv_args& a, hipStream_t s) {
   const size_t lds = (size_t)a.K * sizeof(float);
+  const int64_t units = a.epi == MTJ_EPI_INPROJ ? a.N / 2 : a.N;
+  int64_t grid = 256;                                       // one workgroup per CU
+  if (grid > (units + 15) / 16) grid = (units + 15) / 16;   // at least one unit per wavefront
+  if (grid < 1) grid = 1;
+  const int64_t upw = a.epi == MTJ_EPI_INPROJ ? 2 : 1;
+  while ((units + grid * 16 - 1) / (grid * 16) * upw > 62) grid *= 2;   // a lane per row: <= 64 rows per wavefront
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<T, R, U>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<T, U>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256);
     if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_gemv: hipFuncSetAttribute: %s", hipGetErrorString(e));
     attr_set = true;
   }
-  gemv_kernel<T, R, U><<<grid, waves * 64, lds, s>>>(a);
+  gemv_kernel<T, U><<<(unsigned)grid, 1024, lds, s>>>(a);
   return mtj_check_launch("mtj_gemv");
 }
 
 template <typename T>
 int dispatch(const gemv_args& a, hipStream_t s) {
-  // Small K (x fits LDS many times over): 4 wavefronts x 4 rows, so thousands of workgroups.
-  // Large K (the 80 KiB out|fc_out input): one 16-wavefront workgroup per CU, the rows split evenly.
-  if (a.K * 4 <= 40 * 1024) {
-    if (a.N >= 16 * 1024) return launch<T, 4, 4>(a, 4, s);
-    return launch<T, 2, 8>(a, 4, s);
-  }
-  if (a.epi == MTJ_EPI_INPROJ) return launch<T, 2, 8>(a, 16, s);
-  if (a.N >= 16 * 512) return launch<T, 2, 8>(a, 16, s);
-  return launch<T, 1, 8>(a, 16, s);
+  return launch<T, 8>(a, s);
 }
 
 }  // namespace

@@ -7,17 +7,40 @@ namespace {
 
 constexpr int SNT = 1024;  // threads per row
 
+// x_next[b, :] = W[token, :] + bias, by the whole workgroup (token is uniform)
+__device__ __forceinline__ void embed_next(const mtj_next_embed& ne, int b, int V, int token) {
+  if (!ne.w) return;
+  const bool hit = (uint32_t)token < (uint32_t)V;
+  float* xo = ne.x_next + (int64_t)b * ne.d;
+  for (int64_t c = threadIdx.x; c < ne.d; c += blockDim.x) {
+    float w = 0.f;
+    if (hit) w = ne.dtype == MTJ_F32 ? reinterpret_cast<const float*>(ne.w)[(int64_t)token * ne.d + c]
+                                     : elem<bf16_t>::load(reinterpret_cast<const bf16_t*>(ne.w) + (int64_t)token * ne.d + c);
+    xo[c] = w + ne.bias[c];
+  }
+}
+
 // ---------------------------------------------------------------- greedy
 __global__ __launch_bounds__(SNT) void greedy_kernel(const float* __restrict__ logits, int V, int32_t* __restrict__ tok,
                                                      int32_t* __restrict__ out_tokens, int64_t ld_tokens,
-                                                     int32_t* __restrict__ pos, const int32_t* __restrict__ pos_start) {
+                                                     int32_t* __restrict__ pos, const int32_t* __restrict__ pos_start,
+                                                     const mtj_next_embed ne) {
   __shared__ float sv[SNT / 64];
   __shared__ int si[SNT / 64];
+  __shared__ int chosen;
   const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* row = logits + (int64_t)b * V;
   float best = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = tid; i < V; i += SNT) {
+  const int V4 = ((reinterpret_cast<uintptr_t>(row) & 15u) == 0) ? (V & ~3) : 0;   // float4 body when aligned
+  for (int i = tid * 4; i < V4; i += SNT * 4) {
+    const floatx4 v = *reinterpret_cast<const floatx4*>(row + i);
+    if (v.x > best) { best = v.x; bi = i; }          // indices grow, so '>' keeps the lowest id of a tie
+    if (v.y > best) { best = v.y; bi = i + 1; }
+    if (v.z > best) { best = v.z; bi = i + 2; }
+    if (v.w > best) { best = v.w; bi = i + 3; }
+  }
+  for (int i = V4 + tid; i < V; i += SNT) {
     const float v = row[i];
     if (v > best || (v == best && i < bi)) { best = v; bi = i; }
   }
@@ -37,7 +60,10 @@ __global__ __launch_bounds__(SNT) void greedy_kernel(const float* __restrict__ l
     tok[b] = bi;
     if (out_tokens) out_tokens[(int64_t)b * ld_tokens + (pos[b] - pos_start[b])] = bi;
     pos[b] += 1;
+    chosen = bi;
   }
+  __syncthreads();
+  embed_next(ne, b, V, chosen);
 }
 
 // ---------------------------------------------------------------- nucleus
@@ -123,9 +149,10 @@ __global__ __launch_bounds__(SNT) void nucleus_kernel(const float* __restrict__ 
                                                       int64_t ld_tokens, int32_t* __restrict__ pos,
                                                       const int32_t* __restrict__ pos_start,
                                                       uint8_t* __restrict__ keep_mask, float* __restrict__ filtered,
-                                                      float* __restrict__ fsorted) {
+                                                      float* __restrict__ fsorted, const mtj_next_embed ne) {
   __shared__ double sh[SNT / 64];
   __shared__ int sh_i[SNT / 64];
+  __shared__ int chosen;
   const int b = blockIdx.x, tid = threadIdx.x;
   const uint64_t* srt = sorted + (int64_t)b * V;
   float* fs = fsorted + (int64_t)b * V;           // filtered logits in sorted order
@@ -189,7 +216,10 @@ __global__ __launch_bounds__(SNT) void nucleus_kernel(const float* __restrict__ 
     tok[b] = id;
     if (out_tokens) out_tokens[(int64_t)b * ld_tokens + step] = id;
     pos[b] += 1;
+    chosen = id;
   }
+  __syncthreads();
+  embed_next(ne, b, V, chosen);
 }
 
 struct sample_layout {
@@ -213,11 +243,23 @@ sample_layout layout(int64_t B, int64_t V) {
 
 }  // namespace
 
+static int check_next(const mtj_next_embed* next, mtj_next_embed* ne, const char* who) {
+  *ne = mtj_next_embed{nullptr, nullptr, nullptr, 0, 0};
+  if (!next || !next->w) return MTJ_OK;
+  MTJ_REQUIRE(next->bias && next->x_next && next->d > 0 && (next->dtype == MTJ_F32 || next->dtype == MTJ_BF16), MTJ_EINVAL,
+              "%s: incomplete next-step embedding", who);
+  *ne = *next;
+  return MTJ_OK;
+}
+
 extern "C" int mtj_sample_greedy(const float* logits, int64_t B, int64_t V, int32_t* tok, int32_t* out_tokens,
-                                 int64_t ld_tokens, int32_t* pos, const int32_t* pos_start, void* stream) {
+                                 int64_t ld_tokens, int32_t* pos, const int32_t* pos_start, const mtj_next_embed* next,
+                                 void* stream) {
   MTJ_REQUIRE(logits && tok && pos && pos_start, MTJ_EINVAL, "mtj_sample_greedy: null pointer");
   MTJ_REQUIRE(B > 0 && V > 0 && V < (1ll << 31), MTJ_EINVAL, "mtj_sample_greedy: bad shape");
-  greedy_kernel<<<(unsigned)B, SNT, 0, (hipStream_t)stream>>>(logits, (int)V, tok, out_tokens, ld_tokens, pos, pos_start);
+  mtj_next_embed ne;
+  if (int rc = check_next(next, &ne, "mtj_sample_greedy")) return rc;
+  greedy_kernel<<<(unsigned)B, SNT, 0, (hipStream_t)stream>>>(logits, (int)V, tok, out_tokens, ld_tokens, pos, pos_start, ne);
   return mtj_check_launch("mtj_sample_greedy");
 }
 
@@ -226,12 +268,15 @@ extern "C" int64_t mtj_sample_work_bytes(int64_t B, int64_t V) { return (int64_t
 extern "C" int mtj_sample_nucleus(const float* logits, int64_t B, int64_t V, const double* top_p, const double* temp,
                                   const int32_t* top_k, const double* uniforms, int64_t ld_u, int32_t* tok,
                                   int32_t* out_tokens, int64_t ld_tokens, int32_t* pos, const int32_t* pos_start,
-                                  uint8_t* keep_mask, float* filtered, void* work, void* stream) {
+                                  uint8_t* keep_mask, float* filtered, void* work, const mtj_next_embed* next,
+                                  void* stream) {
   MTJ_REQUIRE(logits && top_p && temp && uniforms && tok && pos && pos_start && work, MTJ_EINVAL,
               "mtj_sample_nucleus: null pointer");
   MTJ_REQUIRE(B > 0 && V > 0 && V <= 65536 && B * V < (1ll << 31), MTJ_EINVAL,
               "mtj_sample_nucleus: V=%lld must be <= 65536 (token id shares the sort key)", (long long)V);
   MTJ_REQUIRE((reinterpret_cast<uintptr_t>(work) & 255u) == 0, MTJ_EALIGN, "mtj_sample_nucleus: work must be 256-byte aligned");
+  mtj_next_embed ne;
+  if (int rc = check_next(next, &ne, "mtj_sample_nucleus")) return rc;
   hipStream_t s = (hipStream_t)stream;
   const sample_layout L = layout(B, V);
   unsigned char* w = reinterpret_cast<unsigned char*>(work);
@@ -252,6 +297,6 @@ extern "C" int mtj_sample_nucleus(const float* logits, int64_t B, int64_t V, con
                                               off + 1, 0, 48, s, false);
   if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_sample_nucleus: sort: %s", hipGetErrorString(e));
   nucleus_kernel<<<(unsigned)B, SNT, 0, s>>>(logits, kout, (int)V, top_p, temp, top_k, uniforms, ld_u, tok, out_tokens,
-                                             ld_tokens, pos, pos_start, keep_mask, filtered, fsorted);
+                                             ld_tokens, pos, pos_start, keep_mask, filtered, fsorted, ne);
   return mtj_check_launch("mtj_sample_nucleus");
 }

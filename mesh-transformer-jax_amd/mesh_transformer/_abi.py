@@ -28,6 +28,11 @@ class InProj(C.Structure):
     ]
 
 
+class NextEmbed(C.Structure):
+    """mtj_next_embed"""
+    _fields_ = [("w", _p), ("bias", _p), ("x_next", _p), ("d", _i64), ("dtype", C.c_int32)]
+
+
 # name -> (restype, argtypes); one entry per declaration in mtj_abi.h
 SIGNATURES = {
     "mtj_version": (_i32, []),
@@ -40,9 +45,10 @@ SIGNATURES = {
     "mtj_attn_prefill": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64, _i32, _p]),
     "mtj_attn_decode_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "mtj_attn_decode": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _i32, _i32, _p, _p]),
-    "mtj_sample_greedy": (_i32, [_p, _i64, _i64, _p, _p, _i64, _p, _p, _p]),
+    "mtj_sample_greedy": (_i32, [_p, _i64, _i64, _p, _p, _i64, _p, _p, C.POINTER(NextEmbed), _p]),
     "mtj_sample_work_bytes": (_i64, [_i64, _i64]),
-    "mtj_sample_nucleus": (_i32, [_p, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p, _p]),
+    "mtj_sample_nucleus": (_i32, [_p, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p,
+                                 C.POINTER(NextEmbed), _p]),
 }
 
 _lib = None

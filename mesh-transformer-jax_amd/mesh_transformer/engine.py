@@ -17,7 +17,7 @@ import numpy as np
 import torch
 
 from . import _abi
-from ._abi import BF16, EPI_INPROJ, EPI_RESID, EPI_STORE, F32, InProj, check, ptr
+from ._abi import BF16, EPI_INPROJ, EPI_RESID, EPI_STORE, F32, InProj, NextEmbed, check, ptr
 
 ROOT = "causal_transformer_shard/~/"
 
@@ -124,7 +124,7 @@ class Session:
         self.act = torch.zeros(B, d + F, dtype=act_t, device=dev)
         self.q = torch.empty(B, H, dh, dtype=torch.float32, device=dev)
         self.logits = torch.empty(B, V, dtype=torch.float32, device=dev)
-        self.attn_work = torch.empty(max(L.mtj_attn_decode_work_bytes(B, H, dh, Tcap), 256), dtype=torch.uint8, device=dev)
+        self.attn_work = torch.zeros(max(L.mtj_attn_decode_work_bytes(B, H, dh, Tcap), 256), dtype=torch.uint8, device=dev)
         self.sample_work = None
         self.tok = torch.zeros(B, dtype=torch.int32, device=dev)
         self.pos = torch.zeros(B, dtype=torch.int32, device=dev)
@@ -192,11 +192,25 @@ class Engine:
         check(L.mtj_gemm(ptr(act), d + F, ptr(w.w_out[i]), ptr(w.b2[i]), M, d, d + F, w.dtype, EPI_RESID,
                          ptr(x), d, F32, None, s))
 
+    def embed_tok(self, ses):
+        """x = EmbeddingShard(tok) for the decode step that follows."""
+        w = self.w
+        check(_abi.lib().mtj_embed(ptr(ses.tok), ses.B, ptr(w.we), ptr(w.be), w.V, w.d, w.dtype, ptr(ses.x),
+                                   _abi.stream_handle()))
+
+    def _next(self, ses, fuse):
+        if not fuse:
+            return None
+        w = self.w
+        ne = NextEmbed()
+        ne.w, ne.bias, ne.x_next, ne.d, ne.dtype = ptr(w.we), ptr(w.be), ptr(ses.x), w.d, w.dtype
+        return C.byref(ne)
+
     def decode_model(self, ses):
-        """generate_once (transformer_shard.py:97-115): tok -> logits, K/V window updated in place."""
+        """generate_once (transformer_shard.py:97-115) from the embedded token in ses.x to the logits; the K/V
+        window is updated in place."""
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()
         B, d, F, V = ses.B, w.d, w.F, w.V
-        check(L.mtj_embed(ptr(ses.tok), B, ptr(w.we), ptr(w.be), V, d, w.dtype, ptr(ses.x), s))
         for i in w.layer_ids:
             self.layer_decode(ses, i)
         if ses.gemv_path:
@@ -228,18 +242,20 @@ class Engine:
             check(L.mtj_gemm(ptr(ses.act), d + F, ptr(w.w_out[i]), ptr(w.b2[i]), B, d, d + F, w.dtype, EPI_RESID,
                              ptr(ses.x), d, F32, None, s))
 
-    def sample_greedy(self, ses, out_tokens):
+    def sample_greedy(self, ses, out_tokens, embed_next=True):
         check(_abi.lib().mtj_sample_greedy(ptr(ses.logits), ses.B, self.w.V, ptr(ses.tok), ptr(out_tokens),
-                                           out_tokens.shape[1], ptr(ses.pos), ptr(ses.pos_start), _abi.stream_handle()))
+                                           out_tokens.shape[1], ptr(ses.pos), ptr(ses.pos_start),
+                                           self._next(ses, embed_next), _abi.stream_handle()))
 
-    def sample_nucleus(self, ses, out_tokens, top_p, temp, top_k, uniforms, keep_mask=None, filtered=None):
+    def sample_nucleus(self, ses, out_tokens, top_p, temp, top_k, uniforms, keep_mask=None, filtered=None,
+                       embed_next=True):
         L = _abi.lib()
         if ses.sample_work is None:
             ses.sample_work = torch.empty(L.mtj_sample_work_bytes(ses.B, self.w.V), dtype=torch.uint8, device=self.device)
         check(L.mtj_sample_nucleus(ptr(ses.logits), ses.B, self.w.V, ptr(top_p), ptr(temp), ptr(top_k), ptr(uniforms),
                                    uniforms.shape[1], ptr(ses.tok), ptr(out_tokens), out_tokens.shape[1], ptr(ses.pos),
                                    ptr(ses.pos_start), ptr(keep_mask), ptr(filtered), ptr(ses.sample_work),
-                                   _abi.stream_handle()))
+                                   self._next(ses, embed_next), _abi.stream_handle()))
 
     # ------------------------------------------------------------------ sessions
     def session(self, B, Tcap, Tp_max, max_pos):

@@ -46,7 +46,7 @@ def _run(logits, top_p, temp, top_k, u, want_filtered, want_mask):
         mask = torch.empty(R, V, dtype=torch.uint8, device=dev) if want_mask else None
         work = torch.empty(L.mtj_sample_work_bytes(R, V), dtype=torch.uint8, device=dev)
         check(L.mtj_sample_nucleus(ptr(lg), R, V, ptr(tp), ptr(tm), ptr(tk), ptr(uu), 1, ptr(tok), None, 0, ptr(pos),
-                                   ptr(pos_start), ptr(mask), ptr(filtered), ptr(work), _abi.stream_handle()))
+                                   ptr(pos_start), ptr(mask), ptr(filtered), ptr(work), None, _abi.stream_handle()))
         torch.cuda.current_stream().synchronize()
     conv = (lambda t: None if t is None else t.cpu().numpy()) if is_np else (lambda t: t)
     return conv(tok), conv(filtered), conv(mask)
@@ -89,7 +89,7 @@ def greedy_sample(key, logits, _, **unused):
     with torch.cuda.device(dev):
         tok = torch.zeros(R, dtype=torch.int32, device=dev)
         pos = torch.zeros(R, dtype=torch.int32, device=dev)
-        check(L.mtj_sample_greedy(ptr(lg), R, V, ptr(tok), None, 0, ptr(pos), ptr(pos.clone()), _abi.stream_handle()))
+        check(L.mtj_sample_greedy(ptr(lg), R, V, ptr(tok), None, 0, ptr(pos), ptr(pos.clone()), None, _abi.stream_handle()))
         torch.cuda.current_stream().synchronize()
     return (tok.cpu().numpy().astype(np.uint32) if is_np else tok), None
 

@@ -169,7 +169,8 @@ class CausalTransformer:
             if Tp > 0:
                 eng.prefill(ses, rect, Tp)
             t1 = clock() if timing is not None else 0.0
-            # --- decode
+            # --- decode: the samplers also embed the token they choose, so only the first step needs this
+            eng.embed_tok(ses)
             if kind is None:
                 self._decode_host_sampler(eng, ses, G, sampler, opts, logits_out)
             elif timing is None:
@@ -248,6 +249,8 @@ class CausalTransformer:
         sampler(key, logits[1, V], sampler_input, **options_of_this_sequence) -> (token[1], info)."""
         B = ses.B
         for t in range(G):
+            if t:
+                eng.embed_tok(ses)
             eng.decode_model(ses)
             lg = ses.logits.cpu().numpy()
             if logits_out is not None:

@@ -340,7 +340,7 @@ def test_attn_decode_window(L, dt, dh, H, Tcap, positions):
     kc = torch.randn(B, H, Tcap, dh, generator=g).to(TD[dt]).to(DEV)
     vc = torch.randn(B, H, Tcap, dh, generator=g).to(TD[dt]).to(DEV)
     pos = torch.tensor(positions, dtype=torch.int32, device=DEV)
-    work = torch.empty(L.mtj_attn_decode_work_bytes(B, H, dh, Tcap), dtype=torch.uint8, device=DEV)
+    work = torch.zeros(L.mtj_attn_decode_work_bytes(B, H, dh, Tcap), dtype=torch.uint8, device=DEV)
     out = torch.zeros(B, H * dh + 8, device=DEV)
     a.check(L.mtj_attn_decode(a.ptr(q), a.ptr(kc), a.ptr(vc), a.ptr(pos), B, H, Tcap, dh, a.ptr(out), H * dh + 8, 0,
                               a.dtype_code(TD[dt]), a.ptr(work), S()))
@@ -368,7 +368,7 @@ def _sample(L, logits, top_p, temp, top_k, u):
     work = torch.empty(L.mtj_sample_work_bytes(R, V), dtype=torch.uint8, device=DEV)
     tp, tm = f64(top_p), f64(temp)
     a.check(L.mtj_sample_nucleus(a.ptr(lg), R, V, a.ptr(tp), a.ptr(tm), a.ptr(tk), a.ptr(uu), 1, a.ptr(tok), None, 0,
-                                 a.ptr(pos), a.ptr(pos_start), a.ptr(mask), a.ptr(filt), a.ptr(work), S()))
+                                 a.ptr(pos), a.ptr(pos_start), a.ptr(mask), a.ptr(filt), a.ptr(work), None, S()))
     torch.cuda.synchronize()
     assert torch.all(pos == 1)
     return tok.cpu().numpy(), mask.cpu().numpy().astype(bool), filt.cpu().numpy()
@@ -414,8 +414,14 @@ def test_greedy_lowest_index_on_ties(L):
     pos = torch.tensor([4, 5, 6], dtype=torch.int32, device=DEV)
     pos_start = torch.tensor([4, 4, 4], dtype=torch.int32, device=DEV)
     out = torch.full((3, 4), -1, dtype=torch.int32, device=DEV)
-    a.check(L.mtj_sample_greedy(a.ptr(lg), 3, V, a.ptr(tok), a.ptr(out), 4, a.ptr(pos), a.ptr(pos_start), S()))
+    W = (torch.randn(V, 96) * 0.02).to(torch.bfloat16).to(DEV)
+    bias = torch.randn(96).to(DEV)
+    xn = torch.zeros(3, 96, device=DEV)
+    ne = a.NextEmbed()
+    ne.w, ne.bias, ne.x_next, ne.d, ne.dtype = a.ptr(W), a.ptr(bias), a.ptr(xn), 96, 1
+    a.check(L.mtj_sample_greedy(a.ptr(lg), 3, V, a.ptr(tok), a.ptr(out), 4, a.ptr(pos), a.ptr(pos_start), C.byref(ne), S()))
     torch.cuda.synchronize()
     assert tok.tolist() == [777, V - 1, 0]
     assert out.tolist() == [[777, -1, -1, -1], [-1, V - 1, -1, -1], [-1, -1, 0, -1]]
     assert pos.tolist() == [5, 6, 7]
+    assert torch.equal(xn, W[tok.long()].float() + bias)      # the chosen token's embedding, for the next step

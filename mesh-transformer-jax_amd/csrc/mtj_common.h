@@ -75,11 +75,12 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-// jax.nn.gelu(approximate=True): 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
+// jax.nn.gelu(approximate=True): 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3).
+// 0.5 (1 + tanh(u)) = 1 / (1 + exp(-2u)); evaluated with the hardware exp2 and reciprocal (a few ulp).
 __device__ __forceinline__ float gelu_tanh(float x) {
   const float c = 0.7978845608028654f;
-  float u = c * (x + 0.044715f * x * x * x);
-  return 0.5f * x * (1.0f + tanhf(u));
+  const float u = c * (x + 0.044715f * x * x * x);
+  return __fdividef(x, 1.0f + __expf(-2.0f * u));
 }
 
 // ---------------------------------------------------------------- fused input-projection epilogue

@@ -1,8 +1,9 @@
 // MFMA GEMM for prefill and batched decode: C[M, N] = A[M, K] x W[N, K]^T with fused epilogues.
 // Both operands are K-contiguous, are staged global -> registers -> LDS (padded rows, so that the
-// 16-byte fragment reads of a 32x32 MFMA hit 64 distinct banks) and double-buffered; accumulation is
+// 16-byte fragment reads of a 32x32 MFMA hit distinct banks) and double-buffered; accumulation is
 // float32.  bf16 uses v_mfma_f32_32x32x16_bf16, float32 uses v_mfma_f32_32x32x2_f32 (true fp32).
 #include "mtj_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -46,7 +47,6 @@ struct gemm_args {
   const void* W;
   const float* bias;
   int M, N, K;
-  int epi;
   void* out;
   int64_t ldo;
   int out_dtype;
@@ -54,8 +54,38 @@ struct gemm_args {
   mtj_inproj ip;
 };
 
-// Workgroup tile (WAVES_M*WM*32) x (WAVES_N*WN*32), K step BK elements.
-template <typename T, int WAVES_M, int WAVES_N, int WM, int WN, int BK>
+template <int DT>
+__device__ __forceinline__ void store_t(void* base, int64_t idx, float v) {
+  if (DT == MTJ_F32) reinterpret_cast<float*>(base)[idx] = v;
+  else reinterpret_cast<uint16_t*>(base)[idx] = (uint16_t)f32_to_bf16_bits(v);
+}
+
+// 16 consecutive elements, 16-byte vector stores (idx is a multiple of 16 elements, base 16-byte aligned)
+__device__ __forceinline__ void store16(void* base, int64_t idx, const float* v, int dtype) {
+  if (dtype == MTJ_F32) {
+    floatx4* p = reinterpret_cast<floatx4*>(reinterpret_cast<float*>(base) + idx);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) p[q] = floatx4{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+  } else {
+    uint32x4* p = reinterpret_cast<uint32x4*>(reinterpret_cast<uint16_t*>(base) + idx);
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      p[q] = uint32x4{pack_bf16x2(v[8 * q], v[8 * q + 1]), pack_bf16x2(v[8 * q + 2], v[8 * q + 3]),
+                      pack_bf16x2(v[8 * q + 4], v[8 * q + 5]), pack_bf16x2(v[8 * q + 6], v[8 * q + 7])};
+  }
+}
+
+// compile-time loop over the accumulator tiles (i, j) of a wavefront: the indices must be constants for the
+// accumulators to stay in registers
+template <int I, int J, int WM, int WN, class F>
+__device__ __forceinline__ void for_tiles(F&& f) {
+  f(std::integral_constant<int, I>{}, std::integral_constant<int, J>{});
+  if constexpr (I + 1 < WM) for_tiles<I + 1, J, WM, WN>(f);
+  else if constexpr (J + 1 < WN) for_tiles<0, J + 1, WM, WN>(f);
+}
+
+// Workgroup tile (WAVES_M*WM*32) x (WAVES_N*WN*32), K step BK elements, epilogue EPI.
+template <typename T, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_args a) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
@@ -94,22 +124,27 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
   const T* __restrict__ A = reinterpret_cast<const T*>(a.A);
   const T* __restrict__ W = reinterpret_cast<const T*>(a.W);
 
+  // per-thread global source pointers (rows beyond M / N are clamped: their products are never stored)
+  const T* ga[A_CHUNKS];
+  const T* gb[B_CHUNKS];
+#pragma unroll
+  for (int i = 0; i < A_CHUNKS; ++i) {
+    const int c = i * NT + tid, row = c / CPR, cc = c % CPR;
+    const int m = (m0 + row < a.M) ? m0 + row : a.M - 1;
+    ga[i] = A + (int64_t)m * a.lda + cc * EPC;
+  }
+#pragma unroll
+  for (int i = 0; i < B_CHUNKS; ++i) {
+    const int c = i * NT + tid, row = c / CPR, cc = c % CPR;
+    const int n = (n0 + row < a.N) ? n0 + row : a.N - 1;
+    gb[i] = W + (int64_t)n * a.K + cc * EPC;
+  }
   uint32x4 ra[A_CHUNKS], rb[B_CHUNKS];
   auto load_global = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      const int c = i * NT + tid, row = c / CPR, cc = c % CPR;
-      const int m = m0 + row;
-      ra[i] = (m < a.M) ? *reinterpret_cast<const uint32x4*>(A + (int64_t)m * a.lda + k0 + cc * EPC)
-                        : uint32x4{0, 0, 0, 0};
-    }
+    for (int i = 0; i < A_CHUNKS; ++i) ra[i] = *reinterpret_cast<const uint32x4*>(ga[i] + k0);
 #pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-      const int c = i * NT + tid, row = c / CPR, cc = c % CPR;
-      const int n = n0 + row;
-      rb[i] = (n < a.N) ? *reinterpret_cast<const uint32x4*>(W + (int64_t)n * a.K + k0 + cc * EPC)
-                        : uint32x4{0, 0, 0, 0};
-    }
+    for (int i = 0; i < B_CHUNKS; ++i) rb[i] = *reinterpret_cast<const uint32x4*>(gb[i] + k0);
   };
   auto store_lds = [&](int buf) {
 #pragma unroll
@@ -158,54 +193,134 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
   }
 
   // ---- epilogue.  Accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32].
+  if (EPI == MTJ_EPI_INPROJ) {
+    // Each 32x32 accumulator tile goes through a private LDS patch of its wavefront and comes back with one
+    // lane owning 16 consecutive columns of one row: rotary pairs are then lane-local and every destination
+    // (q, K/V window, gelu(fc_in)) gets 32- or 64-byte stores.  The operand tiles are no longer needed.
+    int* row_b = reinterpret_cast<int*>(smem);
+    int* row_pos = row_b + BM;
+    float* patch = reinterpret_cast<float*>(smem) + 2 * BM + wave * (32 * 33);
+    for (int r = tid; r < BM; r += NT) {
+      const int m = m0 + r;
+      int b = 0, pos = -1;
+      if (m < a.M) {
+        b = m / a.ip.Tp;
+        pos = a.ip.pos0[b] + (m - b * a.ip.Tp);
+      }
+      row_b[r] = b;
+      row_pos[r] = pos;
+    }
+    __syncthreads();
+    const int d = a.ip.n_heads * a.ip.d_head, dh = a.ip.d_head, rd = a.ip.rotary_dims, Tp = a.ip.Tp;
+    const int prow = lane >> 1, pcol = (lane & 1) * 16;     // my row / first column inside a tile
+    for_tiles<0, 0, WM, WN>([&](auto I_, auto J_) {
+      constexpr int i = decltype(I_)::value, j = decltype(J_)::value;
+      const int nb = n0 + (wn * WN + j) * 32;               // first column of this tile (tile-uniform facts below)
+      const bool is_fc = nb >= 3 * d;
+      const int seg = is_fc ? 3 : nb / d;                   // 0 q, 1 v, 2 k
+      const int c0 = nb - seg * d + pcol;                   // my first column inside the segment
+      const int h = c0 / dh, e0 = c0 - h * dh;
+      const bool n_ok = nb + pcol < a.N;                    // N is a multiple of 16 columns here
+      {
 #pragma unroll
-  for (int i = 0; i < WM; ++i)
+        for (int v = 0; v < 16; ++v) patch[(8 * (v / 4) + 4 * fg + (v % 4)) * 33 + fr] = acc[i][j][v];
+        __builtin_amdgcn_wave_barrier();
+        float val[16];
 #pragma unroll
-    for (int j = 0; j < WN; ++j) {
-      const int n = n0 + (wn * WN + j) * 32 + fr;
-      const float bias = (a.bias && a.epi != MTJ_EPI_INPROJ && n < a.N) ? a.bias[n] : 0.f;
+        for (int k = 0; k < 16; ++k) val[k] = patch[prow * 33 + pcol + k];
+        __builtin_amdgcn_wave_barrier();
+        const int r = (wm * WM + i) * 32 + prow;
+        const int m = m0 + r;
+        if (m < a.M && n_ok) {
+          if (is_fc) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m0 + (wm * WM + i) * 32 + 8 * (v / 4) + 4 * fg + (v % 4);
-        const float own = acc[i][j][v];
-        if (a.epi == MTJ_EPI_INPROJ) {
-          const float partner = __shfl_xor(own, 1);
-          if (m < a.M && n < a.N) inproj_store(a.ip, a.bias, a.kv_dtype, m, n, own, partner);
-        } else if (m < a.M && n < a.N) {
-          const int64_t idx = (int64_t)m * a.ldo + n;
-          if (a.epi == MTJ_EPI_STORE) {
-            store_as(a.out, idx, own + bias, a.out_dtype);
+            for (int k = 0; k < 16; ++k) val[k] = gelu_tanh(val[k] + a.bias[c0 + k]);
+            store16(a.ip.act, (int64_t)m * a.ip.ld_act + d + c0, val, a.ip.act_dtype);
           } else {
-            float* o = reinterpret_cast<float*>(a.out);
-            o[idx] += own + bias;
+            const int pos = row_pos[r];
+            if (pos >= 0) {
+              const int b = row_b[r];
+              if (seg != 1 && e0 < rd) {                    // rd is a multiple of 16 (checked on the host)
+                const int pp = pos < a.ip.max_pos ? pos : a.ip.max_pos - 1;
+                const float* sp = a.ip.sin_tab + (int64_t)pp * (rd / 2) + (e0 >> 1);
+                const float* cp = a.ip.cos_tab + (int64_t)pp * (rd / 2) + (e0 >> 1);
+#pragma unroll
+                for (int k = 0; k < 16; k += 2) {
+                  const float sn = sp[k >> 1], cs = cp[k >> 1];
+                  const float x0 = val[k], x1 = val[k + 1];
+                  val[k] = x0 * cs - x1 * sn;
+                  val[k + 1] = x1 * cs + x0 * sn;
+                }
+              }
+              const int64_t bh = (int64_t)b * a.ip.n_heads + h;
+              if (seg == 0) {
+                store16(a.ip.q, (bh * Tp + (m - b * Tp)) * dh + e0, val, a.ip.q_dtype);
+              } else {
+                const int slot = pos % a.ip.Tcap;
+                store16(seg == 1 ? a.ip.v_cache : a.ip.k_cache, (bh * a.ip.Tcap + slot) * dh + e0, val, a.kv_dtype);
+                if (seg == 1 && a.ip.v_t && pos < a.ip.ldvt) {
+#pragma unroll
+                  for (int k = 0; k < 16; ++k) store_as(a.ip.v_t, (bh * dh + e0 + k) * a.ip.ldvt + pos, val[k], a.kv_dtype);
+                }
+              }
+            }
           }
         }
       }
-    }
+    });
+  } else {
+    for_tiles<0, 0, WM, WN>([&](auto I_, auto J_) {
+      constexpr int i = decltype(I_)::value, j = decltype(J_)::value;
+      const int n = n0 + (wn * WN + j) * 32 + fr;
+      const bool n_ok = n < a.N;
+      const float bias = (a.bias && n_ok) ? a.bias[n] : 0.f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + (wm * WM + i) * 32 + 8 * (v / 4) + 4 * fg + (v % 4);
+        if (m < a.M && n_ok) {
+          const int64_t idx = (int64_t)m * a.ldo + n;
+          const float val = acc[i][j][v] + bias;
+          if (EPI == MTJ_EPI_RESID) reinterpret_cast<float*>(a.out)[idx] += val;
+          else if (a.out_dtype == MTJ_F32) reinterpret_cast<float*>(a.out)[idx] = val;
+          else reinterpret_cast<uint16_t*>(a.out)[idx] = (uint16_t)f32_to_bf16_bits(val);
+        }
+      }
+    });
+  }
 }
 
-template <typename T, int WAVES_M, int WAVES_N, int WM, int WN, int BK>
+template <typename T, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK>
 int launch(const gemm_args& a, hipStream_t s) {
   constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
   constexpr size_t lds = 2 * (size_t)(BM + BN) * (BK + mma<T>::EPC) * sizeof(T);
   static_assert(lds <= 160 * 1024, "tile does not fit LDS");
+  static_assert(lds >= 2 * BM * sizeof(int) + WAVES_M * WAVES_N * 32 * 33 * sizeof(float), "epilogue scratch does not fit");
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, WAVES_M, WAVES_N, WM, WN, BK>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_gemm: hipFuncSetAttribute: %s", hipGetErrorString(e));
     attr_set = true;
   }
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  gemm_kernel<T, WAVES_M, WAVES_N, WM, WN, BK><<<tiles, WAVES_M * WAVES_N * 64, lds, s>>>(a);
+  gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK><<<tiles, WAVES_M * WAVES_N * 64, lds, s>>>(a);
   return mtj_check_launch("mtj_gemm");
 }
 
+template <typename T, int EPI, int BK>
+int dispatch_tile(const gemm_args& a, hipStream_t s) {
+  if (a.M <= 32) return launch<T, EPI, 1, 4, 1, 2, BK>(a, s);    // 32 x 256: batched decode, weights stream once
+  if (a.M <= 64) return launch<T, EPI, 1, 4, 2, 2, BK>(a, s);    // 64 x 256
+  const int64_t big = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
+  if (big >= 200) return launch<T, EPI, 2, 2, 4, 4, BK>(a, s);   // 256 x 256, wavefront tile 128 x 128
+  return launch<T, EPI, 2, 2, 2, 2, BK>(a, s);                   // 128 x 128
+}
+
 template <typename T, int BK>
-int dispatch(const gemm_args& a, hipStream_t s) {
-  if (a.M <= 32) return launch<T, 1, 4, 1, 2, BK>(a, s);    // 32 x 256: batched decode, weights stream once
-  if (a.M <= 64) return launch<T, 1, 4, 2, 2, BK>(a, s);    // 64 x 256
-  return launch<T, 2, 2, 2, 2, BK>(a, s);                   // 128 x 128
+int dispatch(const gemm_args& a, int epi, hipStream_t s) {
+  if (epi == MTJ_EPI_STORE) return dispatch_tile<T, MTJ_EPI_STORE, BK>(a, s);
+  if (epi == MTJ_EPI_RESID) return dispatch_tile<T, MTJ_EPI_RESID, BK>(a, s);
+  return dispatch_tile<T, MTJ_EPI_INPROJ, BK>(a, s);
 }
 
 }  // namespace
@@ -225,12 +340,13 @@ extern "C" int mtj_gemm(const void* A, int64_t lda, const void* W, const float* 
               "mtj_gemm: A, W and the row stride of A must be 16-byte aligned");
   gemm_args a{};
   a.A = A; a.lda = lda; a.W = W; a.bias = bias; a.M = (int)M; a.N = (int)N; a.K = (int)K;
-  a.epi = epi; a.out = out; a.ldo = ldo; a.out_dtype = out_dtype; a.kv_dtype = dtype;
+  a.out = out; a.ldo = ldo; a.out_dtype = out_dtype; a.kv_dtype = dtype;
   if (epi == MTJ_EPI_INPROJ) {
     MTJ_REQUIRE(ip && bias, MTJ_EINVAL, "mtj_gemm: INPROJ needs ip and the fc_in bias");
     a.ip = *ip;
     const int64_t d = (int64_t)ip->n_heads * ip->d_head;
-    MTJ_REQUIRE(ip->Tp > 0 && M % ip->Tp == 0 && N > 3 * d && N % 2 == 0 && ip->rotary_dims % 2 == 0 &&
+    MTJ_REQUIRE(ip->Tp > 0 && M % ip->Tp == 0 && N > 3 * d && N % 32 == 0 && d % 32 == 0 && ip->d_head % 32 == 0 &&
+                    ip->rotary_dims % 16 == 0 && ip->ld_act % 16 == 0 &&
                     ip->rotary_dims <= ip->d_head && ip->Tcap > 0 && ip->max_pos > 0 && ip->pos0 && ip->sin_tab &&
                     ip->cos_tab && ip->q && ip->k_cache && ip->v_cache && ip->act && ip->ld_act >= N - 2 * d &&
                     (ip->act_dtype == MTJ_F32 || ip->act_dtype == MTJ_BF16) &&
@@ -245,5 +361,5 @@ extern "C" int mtj_gemm(const void* A, int64_t lda, const void* W, const float* 
     return mtj_fail(MTJ_EINVAL, "mtj_gemm: epilogue %d", epi);
   }
   hipStream_t s = (hipStream_t)stream;
-  return dtype == MTJ_BF16 ? dispatch<bf16_t, 64>(a, s) : dispatch<float, 32>(a, s);
+  return dtype == MTJ_BF16 ? dispatch<bf16_t, 64>(a, epi, s) : dispatch<float, 32>(a, epi, s);
 }

@@ -84,16 +84,29 @@ __device__ __forceinline__ void for_tiles(F&& f) {
   else if constexpr (J + 1 < WN) for_tiles<0, J + 1, WM, WN>(f);
 }
 
-// Workgroup tile (WAVES_M*WM*32) x (WAVES_N*WN*32), K step BK elements, epilogue EPI.
-template <typename T, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK>
+template <int S, int NS, class F>
+__device__ __forceinline__ void for_stages(F&& f) {
+  f(std::integral_constant<int, S>{});
+  if constexpr (S + 1 < NS) for_stages<S + 1, NS>(f);
+}
+
+// Workgroup tile (WAVES_M*WM*32) x (WAVES_N*WN*32), K step BK elements, NS register stages, epilogue EPI.
+//
+// Pipeline: k-tile kt is multiplied out of LDS (two buffers) while the loads of k-tiles kt+1 .. kt+NS sit in
+// registers or are still in flight; one k-tile in flight does not cover the load latency of a loaded GPU.
+// Global reads are bounds-checked buffer loads (rows beyond M or N read as zero), whose addressing needs one
+// VGPR per operand: the per-chunk and per-k-tile offsets are scalar.
+template <typename T, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK, int NS>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_args a) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
   constexpr int EPC = mma<T>::EPC;
+  constexpr int ESZ = (int)sizeof(T);
   constexpr int CPR = BK / EPC;          // 16-byte chunks per tile row
   constexpr int LDS_ROW = BK + EPC;      // padded row, elements (row stride 144 B for both types)
   constexpr int A_CHUNKS = BM * CPR / NT, B_CHUNKS = BN * CPR / NT;
-  static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "tile does not divide over threads");
+  constexpr int ROWS_PER_PASS = NT / CPR;   // tile rows covered by one chunk index
+  static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0 && NT % CPR == 0, "tile does not divide over threads");
   static_assert(BK % 16 == 0, "BK must hold whole MFMA k-steps");
 
   extern __shared__ __align__(16) unsigned char smem[];
@@ -121,42 +134,38 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
   const int tn = (pid % (GM * tiles_n)) / gsz;
   const int m0 = tm * BM, n0 = tn * BN;
 
-  const T* __restrict__ A = reinterpret_cast<const T*>(a.A);
-  const T* __restrict__ W = reinterpret_cast<const T*>(a.W);
+  // buffer resources over the rows of this tile: [m0, min(M, m0+BM)) of A and [n0, min(N, n0+BN)) of W
+  const int rows_a = (a.M - m0 < BM) ? a.M - m0 : BM, rows_b = (a.N - n0 < BN) ? a.N - n0 : BN;
+  const T* tile_a = reinterpret_cast<const T*>(a.A) + (int64_t)m0 * a.lda;
+  const T* tile_b = reinterpret_cast<const T*>(a.W) + (int64_t)n0 * a.K;
+  const __amdgpu_buffer_rsrc_t ra_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(tile_a), 0, (int)((((int64_t)rows_a - 1) * a.lda + a.K) * ESZ), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(tile_b), 0, (int)((((int64_t)rows_b - 1) * a.K + a.K) * ESZ), 0x00020000);
+  const int row0 = tid / CPR, cc0 = tid % CPR;
+  const int voff_a = (int)(((int64_t)row0 * a.lda + cc0 * EPC) * ESZ);
+  const int voff_b = (int)(((int64_t)row0 * a.K + cc0 * EPC) * ESZ);
+  const int pass_a = (int)((int64_t)ROWS_PER_PASS * a.lda * ESZ), pass_b = (int)((int64_t)ROWS_PER_PASS * a.K * ESZ);
 
-  // per-thread global source pointers (rows beyond M / N are clamped: their products are never stored)
-  const T* ga[A_CHUNKS];
-  const T* gb[B_CHUNKS];
+  uint32x4 ra[NS][A_CHUNKS], rb[NS][B_CHUNKS];
+  auto load_global = [&](auto ST_, int kt) {
+    constexpr int st = decltype(ST_)::value;
+    const int koff = kt * BK * ESZ;
 #pragma unroll
-  for (int i = 0; i < A_CHUNKS; ++i) {
-    const int c = i * NT + tid, row = c / CPR, cc = c % CPR;
-    const int m = (m0 + row < a.M) ? m0 + row : a.M - 1;
-    ga[i] = A + (int64_t)m * a.lda + cc * EPC;
-  }
+    for (int i = 0; i < A_CHUNKS; ++i)
+      ra[st][i] = __builtin_amdgcn_raw_buffer_load_b128(ra_rsrc, voff_a, koff + i * pass_a, 0);
 #pragma unroll
-  for (int i = 0; i < B_CHUNKS; ++i) {
-    const int c = i * NT + tid, row = c / CPR, cc = c % CPR;
-    const int n = (n0 + row < a.N) ? n0 + row : a.N - 1;
-    gb[i] = W + (int64_t)n * a.K + cc * EPC;
-  }
-  uint32x4 ra[A_CHUNKS], rb[B_CHUNKS];
-  auto load_global = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) ra[i] = *reinterpret_cast<const uint32x4*>(ga[i] + k0);
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) rb[i] = *reinterpret_cast<const uint32x4*>(gb[i] + k0);
+    for (int i = 0; i < B_CHUNKS; ++i)
+      rb[st][i] = __builtin_amdgcn_raw_buffer_load_b128(rb_rsrc, voff_b, koff + i * pass_b, 0);
   };
-  auto store_lds = [&](int buf) {
+  auto store_lds = [&](auto ST_, int buf) {
+    constexpr int st = decltype(ST_)::value;
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      const int c = i * NT + tid, row = c / CPR, cc = c % CPR;
-      *reinterpret_cast<uint32x4*>(As + (buf * BM + row) * LDS_ROW + cc * EPC) = ra[i];
-    }
+    for (int i = 0; i < A_CHUNKS; ++i)
+      *reinterpret_cast<uint32x4*>(As + (buf * BM + row0 + i * ROWS_PER_PASS) * LDS_ROW + cc0 * EPC) = ra[st][i];
 #pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-      const int c = i * NT + tid, row = c / CPR, cc = c % CPR;
-      *reinterpret_cast<uint32x4*>(Bs + (buf * BN + row) * LDS_ROW + cc * EPC) = rb[i];
-    }
+    for (int i = 0; i < B_CHUNKS; ++i)
+      *reinterpret_cast<uint32x4*>(Bs + (buf * BN + row0 + i * ROWS_PER_PASS) * LDS_ROW + cc0 * EPC) = rb[st][i];
   };
 
   floatx16 acc[WM][WN];
@@ -168,12 +177,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int KT = a.K / BK;
-  load_global(0);
-  store_lds(0);
+  // k-tile t lives in register stage t % NS.  Prologue: request k-tiles 0 .. NS-1, park k-tile 0 in LDS,
+  // reuse its stage for k-tile NS.
+  for_stages<0, NS>([&](auto ST_) {
+    if (decltype(ST_)::value < KT) load_global(ST_, decltype(ST_)::value);
+  });
+  store_lds(std::integral_constant<int, 0>{}, 0);
+  if (NS < KT) load_global(std::integral_constant<int, 0>{}, NS);
   __syncthreads();
-  for (int kt = 0; kt < KT; ++kt) {
+
+  // one k-tile; PARK = stage of k-tile kt+1 (a compile-time index: the k loop is unrolled by NS)
+  auto k_tile = [&](int kt, auto PARK_) {
     const int buf = kt & 1;
-    if (kt + 1 < KT) load_global((kt + 1) * BK);
     const T* as = As + (buf * BM + wm * WM * 32 + fr) * LDS_ROW + fg * 8;
     const T* bs = Bs + (buf * BN + wn * WN * 32 + fr) * LDS_ROW + fg * 8;
 #pragma unroll
@@ -188,8 +203,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
 #pragma unroll
         for (int j = 0; j < WN; ++j) mma<T>::run(acc[i][j], fa[i], fb[j]);
     }
-    if (kt + 1 < KT) store_lds(buf ^ 1);
+    if (kt + 1 < KT) store_lds(PARK_, buf ^ 1);
+    if (kt + 1 + NS < KT) load_global(PARK_, kt + 1 + NS);
     __syncthreads();
+  };
+  for (int kt = 0; kt < KT; kt += NS) {
+    for_stages<0, NS>([&](auto S_) {
+      constexpr int s = decltype(S_)::value;
+      if (kt + s < KT) k_tile(kt + s, std::integral_constant<int, (s + 1) % NS>{});
+    });
   }
 
   // ---- epilogue.  Accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32].
@@ -289,7 +311,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
   }
 }
 
-template <typename T, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK>
+template <typename T, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK, int NS>
 int launch(const gemm_args& a, hipStream_t s) {
   constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
   constexpr size_t lds = 2 * (size_t)(BM + BN) * (BK + mma<T>::EPC) * sizeof(T);
@@ -297,23 +319,23 @@ int launch(const gemm_args& a, hipStream_t s) {
   static_assert(lds >= 2 * BM * sizeof(int) + WAVES_M * WAVES_N * 32 * 33 * sizeof(float), "epilogue scratch does not fit");
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK, NS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_gemm: hipFuncSetAttribute: %s", hipGetErrorString(e));
     attr_set = true;
   }
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK><<<tiles, WAVES_M * WAVES_N * 64, lds, s>>>(a);
+  gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK, NS><<<tiles, WAVES_M * WAVES_N * 64, lds, s>>>(a);
   return mtj_check_launch("mtj_gemm");
 }
 
 template <typename T, int EPI, int BK>
 int dispatch_tile(const gemm_args& a, hipStream_t s) {
-  if (a.M <= 32) return launch<T, EPI, 1, 4, 1, 2, BK>(a, s);    // 32 x 256: batched decode, weights stream once
-  if (a.M <= 64) return launch<T, EPI, 1, 4, 2, 2, BK>(a, s);    // 64 x 256
+  if (a.M <= 32) return launch<T, EPI, 1, 4, 1, 2, BK, 2>(a, s);    // 32 x 256: batched decode, weights stream once
+  if (a.M <= 64) return launch<T, EPI, 1, 4, 2, 2, BK, 2>(a, s);    // 64 x 256
   const int64_t big = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
-  if (big >= 200) return launch<T, EPI, 2, 2, 4, 4, BK>(a, s);   // 256 x 256, wavefront tile 128 x 128
-  return launch<T, EPI, 2, 2, 2, 2, BK>(a, s);                   // 128 x 128
+  if (big >= 200) return launch<T, EPI, 2, 4, 4, 2, BK, 2>(a, s);   // 256 x 256, 8 wavefronts of 128 x 64
+  return launch<T, EPI, 2, 2, 2, 2, BK, 2>(a, s);                   // 128 x 128
 }
 
 template <typename T, int BK>
@@ -338,6 +360,8 @@ extern "C" int mtj_gemm(const void* A, int64_t lda, const void* W, const float* 
   MTJ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), MTJ_ELIMIT, "mtj_gemm: dimension too large");
   MTJ_REQUIRE(mtj_aligned16(A) && mtj_aligned16(W) && (lda * esz) % 16 == 0, MTJ_EALIGN,
               "mtj_gemm: A, W and the row stride of A must be 16-byte aligned");
+  MTJ_REQUIRE(256 * lda * esz < (1ll << 31) && 256 * K * esz < (1ll << 31), MTJ_ELIMIT,
+              "mtj_gemm: a 256-row tile of A or W must span less than 2 GiB");
   gemm_args a{};
   a.A = A; a.lda = lda; a.W = W; a.bias = bias; a.M = (int)M; a.N = (int)N; a.K = (int)K;
   a.out = out; a.ldo = ldo; a.out_dtype = out_dtype; a.kv_dtype = dtype;

@@ -27,6 +27,9 @@ for p in (ROOT, os.path.join(ROOT, "mesh-transformer-jax_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK = 8.0e12          # B/s
+# HBM bytes of one launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what
+# the same counter reads for a plain 234,881,024-byte copy (profiles/gemv_inproj_hbm_traffic_pmc.md)
+DOMINANT_KERNEL_TRAFFIC = 235590000
 MFMA_BF16_PEAK = 2.5e15    # flop/s dense
 
 CFG_6B = dict(layers=28, d_model=4096, n_heads=16, n_vocab=50400, norm="layernorm", pe="rotary", pe_rotary_dims=64,
@@ -165,6 +168,36 @@ def cpu_baseline(net, cfg, n_layers=4, steps=8, prompt=512, L=2048):
     }
 
 
+def pmc_probe(dev):
+    """Work for a hardware-counter pass: a device-to-device copy of exactly the size of W_in (the calibration
+    for FETCH_SIZE / WRITE_SIZE), then the dominant GEMV 8 times over two layers' distinct weights."""
+    import ctypes as C
+    import torch
+    from mesh_transformer import _abi, sampling
+    from mesh_transformer._abi import EPI_INPROJ, F32, check, ptr
+    from mesh_transformer.transformer_shard import CausalTransformer
+    cfg = dict(CFG_6B, layers=2, sampler=sampling.greedy_sample)
+    net = CausalTransformer(cfg, synthetic_tree(cfg, 2, dev, torch.bfloat16))
+    eng = net.engine()
+    ses = eng.session(1, 2047, 1, 1024)
+    L, w = _abi.lib(), eng.w
+    src = torch.empty(234881024, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    ses.pos.fill_(600)
+    ses.x.normal_()
+    s = _abi.stream_handle()
+    for rep in range(4):
+        for i in w.layer_ids:
+            ip = eng._inproj(ses, i, 1, ses.pos, ses.q, F32, ses.act, F32, None)
+            check(L.mtj_gemv(ptr(ses.x), ptr(w.ln_s[i]), ptr(w.ln_o[i]), ptr(w.w_in[i]), ptr(w.b1[i]), 3 * w.d + w.F, w.d,
+                             w.dtype, EPI_INPROJ, None, 0, C.byref(ip), s))
+    torch.cuda.synchronize()
+    print("pmc probe done")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -172,6 +205,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=17)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the prefill-layer measurement")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="counter probe for rocprofv3 --pmc: one plain 234,881,024-byte device copy, then 8 launches "
+                         "of the dominant kernel on a 2-layer model of the 6B shape; prints no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the whole model on ONE GPU (no collectives, no sharding); "
@@ -186,6 +222,9 @@ def main():
 
     _abi.lib()
     dev = torch.device("cuda:0")
+    if args.pmc_probe:
+        pmc_probe(dev)
+        return
     cfg = dict(CFG_6B, sampler=sampling.greedy_sample)
     K, W = args.steps, args.warmup
     net = CausalTransformer(cfg, synthetic_tree(cfg, 2, dev, torch.bfloat16))
@@ -207,7 +246,7 @@ def main():
     k_bytes = gemv_inproj_bytes(cfg)
     roofline = {"bound": "hbm", "kernel": "gemv_kernel (LayerNorm + q|v|k|fc_in, N=28672, K=4096, bf16)",
                 "achieved": k_bytes / t_k / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                "frac": k_bytes / t_k / HBM_PEAK, "traffic": None, "bytes_per_launch": k_bytes,
+                "frac": k_bytes / t_k / HBM_PEAK, "traffic": DOMINANT_KERNEL_TRAFFIC, "bytes_per_launch": k_bytes,
                 "avg_launch_us": t_k * 1e6}
 
     d, F, n = cfg["d_model"], 4 * cfg["d_model"], cfg["layers"]

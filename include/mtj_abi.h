@@ -69,7 +69,7 @@ typedef struct {
   void* k_cache;                        /* [B, H, Tcap, dh] dtype, rotated keys                        */
   void* v_cache;                        /* [B, H, Tcap, dh] dtype                                      */
   void* v_t;                            /* optional [B, H, dh, ldvt] dtype: V transposed, for prefill  */
-  int64_t ldvt;                         /* row length of v_t (>= Tp, multiple of 8)                    */
+  int64_t ldvt;                         /* row length of v_t: >= Tp rounded up to a multiple of 64     */
   void* act;                            /* [M, ld_act]: gelu(fc_in) goes to columns [d, d+F)           */
   int64_t ld_act;
   int32_t act_dtype;                    /* MTJ_F32 or MTJ_BF16                                         */
@@ -109,7 +109,8 @@ int mtj_gemv(const float* x, const float* ln_scale, const float* ln_offset, cons
              void* stream);
 
 /* Causal self-attention over a left-padded rectangle (self_attn + masks of get_init_decode_state,
- * layers.py:260-285, 347-366).  q [B,H,Tp,dh], k_cache [B,H,Tcap,dh] (rotated), v_t [B,H,dh,ldvt];
+ * layers.py:260-285, 347-366).  q [B,H,Tp,dh], k_cache [B,H,Tcap,dh] (rotated), v_t [B,H,dh,ldvt] with
+ * ldvt >= Tp rounded up to a multiple of 64 (columns beyond the last key may hold anything);
  * out[m, h*dh + c] with row stride ld_out, dtype.  Scores are divided by sqrt(dh) after the dot;
  * masked keys contribute exactly 0 (exp(-1e10 - max) underflows in float32).  Padding rows get zeros. */
 int mtj_attn_prefill(const void* q, const void* k_cache, const void* v_t, const int32_t* pos0, int64_t B,

@@ -1,5 +1,6 @@
 // Attention: MFMA flash-style prefill over a left-padded rectangle, and one-token decode over the K/V window.
 #include "mtj_common.h"
+#include <cstdlib>
 
 namespace {
 
@@ -13,6 +14,7 @@ template <> struct mma<bf16_t> {
     f.v = *reinterpret_cast<const bf16x8*>(p);
     return f;
   }
+  __device__ static __forceinline__ void pin(frag& f) { asm volatile("" : "+v"(f.v)); }
   __device__ static __forceinline__ frag from_floats(const float* p) {  // 8 probabilities -> operand
     frag f;
     uint32x4 u;
@@ -38,6 +40,7 @@ template <> struct mma<float> {
     f.v[4] = hi.x; f.v[5] = hi.y; f.v[6] = hi.z; f.v[7] = hi.w;
     return f;
   }
+  __device__ static __forceinline__ void pin(frag&) {}
   __device__ static __forceinline__ frag from_floats(const float* p) {
     frag f;
 #pragma unroll
@@ -52,37 +55,49 @@ template <> struct mma<float> {
 
 // ------------------------------------------------------------------------------------------------
 // Prefill.  Everything is computed transposed so that one lane owns one query: S^T = K Q^T gives each
-// lane (query = lane % 32) sixteen keys of a 32-key tile, the online-softmax state is lane-local, and
+// lane (query = lane % 32) sixteen keys of a 32-key block, the online-softmax state is lane-local, and
 // O^T = V^T P^T is rescaled without any cross-lane traffic.  K rows are fetched in a permuted order so
 // that the sixteen keys a lane ends up with are 8 consecutive ones per MFMA k-step - exactly the
 // operand layout the second MFMA wants for P^T - and V comes pre-transposed ([dh][keys]).
 //
-// Workgroup: 4 wavefronts x 32 queries; K/V tiles of 32 keys staged through LDS.
-template <typename T, int DH>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ kc,
-                                                           const T* __restrict__ vt, const int32_t* __restrict__ pos0,
-                                                           int H, int Tp, int Tcap, int64_t ldvt, T* __restrict__ out,
-                                                           int64_t ld_out) {
+// Workgroup: NW wavefronts x 32 queries; K / V^T tiles of BKV keys are staged global -> registers -> LDS,
+// double-buffered (the loads of tile kt+1 are in flight while tile kt is multiplied).  The softmax runs in
+// the exp2 domain with the hardware exponential; the accumulator is rescaled only when some lane's running
+// maximum actually moved.
+template <typename T, int DH, int NW, int BKV>
+__global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ kc,
+                                                               const T* __restrict__ vt, const int32_t* __restrict__ pos0,
+                                                               int H, int Tp, int Tcap, int64_t ldvt, T* __restrict__ out,
+                                                               int64_t ld_out, int dbg) {
+  constexpr int NT = NW * 64;
+  constexpr int BQ = NW * 32;
   constexpr int EPC = mma<T>::EPC;
   using raw_t = typename mma<T>::raw_t;
-  constexpr int BKV = 32;
   constexpr int KROW = DH + EPC;     // padded K row (elements)
   constexpr int VROW = BKV + EPC;    // padded V^T row
   constexpr int KS = DH / 16;        // MFMA k-steps over the head dim
   constexpr int NBLK = DH / 32;      // 32-wide blocks of the head dim in O^T
-  __shared__ __align__(16) T Ks[BKV * KROW];
-  __shared__ __align__(16) T Vs[DH * VROW];
+  constexpr int KB = BKV / 32;       // 32-key blocks per tile
+  constexpr int CPRK = DH / EPC, CPRV = BKV / EPC;
+  constexpr int K_CHUNKS = BKV * CPRK / NT, V_CHUNKS = DH * CPRV / NT;
+  static_assert(BKV * CPRK % NT == 0 && DH * CPRV % NT == 0, "tile does not divide over threads");
+  extern __shared__ __align__(16) unsigned char smem[];
+  T* Ks = reinterpret_cast<T*>(smem);              // [2][BKV][KROW]
+  T* Vs = Ks + 2 * BKV * KROW;                     // [2][DH][VROW]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 31, fg = lane >> 5;
   const int h = blockIdx.y, b = blockIdx.z;
-  const int qt0 = blockIdx.x * 128;
+  const int qt0 = (gridDim.x - 1 - blockIdx.x) * BQ;   // longest (latest) query blocks are dispatched first
   const int p0 = pos0[b];                       // <= 0: minus the number of padding rows
   const int t = qt0 + wave * 32 + fr;           // this lane's query (rectangle index)
   const int qpos = (t < Tp) ? t + p0 : -1;      // its position; < 0 = padding / out of range
-  const int last_t = (qt0 + 127 < Tp - 1) ? qt0 + 127 : Tp - 1;
+  const int last_t = (qt0 + BQ - 1 < Tp - 1) ? qt0 + BQ - 1 : Tp - 1;
   const int kmax = last_t + p0;                 // last key any query of this workgroup may see
   const int klast = Tp - 1 + p0;                // last key position that exists for this sequence
+  const int wave_last = qt0 + wave * 32 + 31 + p0;   // last key this wavefront may see
+  // first query position of this wavefront if all 32 of its queries are real, else -1 (always mask)
+  const int wave_first = (qt0 + wave * 32 + 31 < Tp) ? qt0 + wave * 32 + p0 : -1;
   const int64_t bh = (int64_t)b * H + h;
 
   // Q fragments (B operand of S^T): lane (query fr, half fg) holds Q[t][ks*16 + fg*8 .. +8)
@@ -91,9 +106,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__
     const int tq = (t < Tp) ? t : Tp - 1;
     const T* qp = q + (bh * Tp + tq) * DH + fg * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = mma<T>::load(qp + ks * 16);
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[ks] = mma<T>::load(qp + ks * 16);
+      mma<T>::pin(qf[ks]);   // or the compiler re-loads Q from global memory inside the key loop
+    }
   }
-  // row fr of the S^T tile is key krow: rows {0-3, 4-7, 8-11, 12-15} <- keys {0-3, 8-11, 4-7, 12-15} (+16)
+  // row fr of an S^T block is key krow: rows {0-3, 4-7, 8-11, 12-15} <- keys {0-3, 8-11, 4-7, 12-15} (+16)
   const int krow = 16 * (fr >> 4) + 8 * ((fr >> 2) & 1) + 4 * ((fr >> 3) & 1) + (fr & 3);
 
   floatx16 o[NBLK];
@@ -101,90 +119,180 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__
   for (int i = 0; i < NBLK; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
-  float mrun = -INFINITY, lrun = 0.f;
-  const float scale = rsqrtf((float)DH);
+  float mrun = -INFINITY, lrun = 0.f;           // running max (log2 units) and sum
+  const float sc2 = rsqrtf((float)DH) * 1.4426950408889634f;   // 1/sqrt(dh) * log2(e)
+
+  // ---- staging
+  uint32x4 rk[K_CHUNKS], rv[V_CHUNKS];
+  // Loads are unconditional: K rows beyond the last key are clamped to it (the causal mask removes them), and a
+  // V^T row is ldvt >= round_up(Tp, BKV) long, so the chunk exists; what it holds beyond the last key is zeroed
+  // in LDS by fix_last_tile (0 x garbage must not become NaN).
+  auto load_tile = [&](int kt) {
+    const int key0 = kt * BKV;
+#pragma unroll
+    for (int i = 0; i < K_CHUNKS; ++i) {
+      const int c = i * NT + tid, row = c / CPRK, cc = c % CPRK;
+      const int key = (key0 + row <= klast) ? key0 + row : klast;
+      rk[i] = *reinterpret_cast<const uint32x4*>(kc + (bh * Tcap + key) * DH + cc * EPC);
+    }
+#pragma unroll
+    for (int i = 0; i < V_CHUNKS; ++i) {
+      const int c = i * NT + tid, row = c / CPRV, cc = c % CPRV;
+      rv[i] = *reinterpret_cast<const uint32x4*>(vt + (bh * DH + row) * ldvt + key0 + cc * EPC);
+    }
+  };
+  auto fix_last_tile = [&](int kt, int buf) {     // workgroup-uniform caller; runs between the store and the barrier
+    const int key0 = kt * BKV;
+    const int nbad = key0 + BKV - 1 - klast;       // columns klast+1-key0 .. BKV-1 of V^T do not exist
+    if (nbad <= 0) return;
+    raw_t* vs = reinterpret_cast<raw_t*>(Vs + buf * DH * VROW);
+    for (int c = tid; c < DH * nbad; c += NT) vs[(c / nbad) * VROW + (BKV - nbad) + (c % nbad)] = (raw_t)0;
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < K_CHUNKS; ++i) {
+      const int c = i * NT + tid, row = c / CPRK, cc = c % CPRK;
+      *reinterpret_cast<uint32x4*>(Ks + (buf * BKV + row) * KROW + cc * EPC) = rk[i];
+    }
+#pragma unroll
+    for (int i = 0; i < V_CHUNKS; ++i) {
+      const int c = i * NT + tid, row = c / CPRV, cc = c % CPRV;
+      *reinterpret_cast<uint32x4*>(Vs + (buf * DH + row) * VROW + cc * EPC) = rv[i];
+    }
+  };
 
   const int ntiles = (kmax >= 0) ? kmax / BKV + 1 : 0;
+  if (ntiles > 0) {
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+    fix_last_tile(0, 0);
+  }
+  __syncthreads();
   for (int kt = 0; kt < ntiles; ++kt) {
+    const int buf = kt & 1;
     const int key0 = kt * BKV;
-    __syncthreads();
-    // ---- stage K tile [32][DH] and V^T tile [DH][32]; keys that do not exist are zero-filled
-    {
-      constexpr int CPRK = DH / EPC;
-      for (int c = tid; c < BKV * CPRK; c += 256) {
-        const int row = c / CPRK, cc = c % CPRK;
-        const int key = key0 + row;
-        uint32x4 val = {0, 0, 0, 0};
-        if (key <= klast) val = *reinterpret_cast<const uint32x4*>(kc + (bh * Tcap + key) * DH + cc * EPC);
-        *reinterpret_cast<uint32x4*>(Ks + row * KROW + cc * EPC) = val;
-      }
-      constexpr int CPRV = BKV / EPC;
-      for (int c = tid; c < DH * CPRV; c += 256) {
-        const int row = c / CPRV, cc = c % CPRV;
-        const int key = key0 + cc * EPC;
-        uint32x4 val = {0, 0, 0, 0};
-        if (key + EPC - 1 <= klast) {
-          val = *reinterpret_cast<const uint32x4*>(vt + (bh * DH + row) * ldvt + key);
-        } else if (key <= klast) {
-          raw_t tmp[EPC];
-          const raw_t* vr = reinterpret_cast<const raw_t*>(vt) + (bh * DH + row) * ldvt + key;
+    if (kt + 1 < ntiles && !(dbg & 8)) load_tile(kt + 1);
+    if (key0 <= wave_last) {      // wave-uniform: tiles entirely above this wavefront's last query are skipped
+      // ---- S^T blocks: rows = (permuted) keys, columns = queries.  The K fragments of k-steps
+      // ks+G .. ks+2G-1 are read from LDS while the MFMAs of k-steps ks .. ks+G-1 run; the KB key blocks
+      // give KB independent accumulation chains.
+      floatx16 s[KB];
 #pragma unroll
-          for (int j = 0; j < EPC; ++j) tmp[j] = (key + j <= klast) ? vr[j] : (raw_t)0;
-          val = *reinterpret_cast<uint32x4*>(tmp);
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[kb][v] = 0.f;
+      {
+        constexpr int G = 2;                       // k-steps per group
+        const T* kp = Ks + (buf * BKV + krow) * KROW + fg * 8;
+        typename mma<T>::frag kf[2][KB][G];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int g = 0; g < G; ++g) kf[0][kb][g] = mma<T>::load(kp + kb * 32 * KROW + g * 16);
+#pragma unroll
+        for (int k0 = 0; k0 < KS; k0 += G) {
+          if (dbg & 2) break;
+          const int cur = (k0 / G) & 1, nxt = cur ^ 1;
+          if (k0 + G < KS) {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+              for (int g = 0; g < G; ++g) kf[nxt][kb][g] = mma<T>::load(kp + kb * 32 * KROW + (k0 + G + g) * 16);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) mma<T>::run(s[kb], kf[cur][kb][g], qf[k0 + g]);
+          __builtin_amdgcn_sched_barrier(0);
         }
-        *reinterpret_cast<uint32x4*>(Vs + row * VROW + cc * EPC) = val;
+      }
+      // register v of block kb is key key0 + kb*32 + 16*(v/8) + 8*fg + v%8
+      float mt = -INFINITY;
+      if (dbg & 4) { mt = s[0][0]; } else
+      if (key0 + BKV - 1 <= wave_first) {   // wave-uniform: the whole tile is below the diagonal for every lane
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            s[kb][v] *= sc2;
+            mt = fmaxf(mt, s[kb][v]);
+          }
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int key = key0 + kb * 32 + 16 * (v / 8) + 8 * fg + (v % 8);
+            s[kb][v] = (key <= qpos) ? s[kb][v] * sc2 : -INFINITY;
+            mt = fmaxf(mt, s[kb][v]);
+          }
+      }
+      mt = fmaxf(mt, __shfl_xor(mt, 32));
+      // The running maximum only moves when a lane's tile maximum exceeds it by more than 2^6: the
+      // probabilities then stay below 64 (harmless in float32 / bf16) and the rescale of the whole
+      // accumulator, which costs as much as the MFMAs of a tile, happens in the first tiles only.
+      if (__any(mt > mrun + 6.0f)) {
+        const float mnew = fmaxf(mrun, mt);
+        const float alpha = (mnew == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(mrun - mnew);   // mrun = -inf -> 0
+        lrun *= alpha;
+#pragma unroll
+        for (int i = 0; i < NBLK; ++i)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
+        mrun = mnew;
+      }
+      const float msafe = (mrun == -INFINITY) ? 0.f : mrun;
+      float lt = 0.f;
+      typename mma<T>::frag pf[KB][2];
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        float p[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          p[v] = __builtin_amdgcn_exp2f(s[kb][v] - msafe);          // masked -> exp2(-inf) = 0
+          lt += p[v];
+        }
+        pf[kb][0] = mma<T>::from_floats(p);
+        pf[kb][1] = mma<T>::from_floats(p + 8);
+      }
+      lt += __shfl_xor(lt, 32);
+      lrun += lt;
+      // ---- O^T += V^T P^T : A = V^T rows (head-dim), B = P^T (keys x queries).  One 16-key k-step at a
+      // time over all NBLK head-dim blocks (NBLK independent accumulators), fragments one k-step ahead.
+      {
+        constexpr int HB = NBLK > 4 ? 4 : NBLK;   // head-dim blocks per pass (bounds the live fragments)
+        const T* vp = Vs + (buf * DH + fr) * VROW + fg * 8;
+#pragma unroll
+        for (int i0 = 0; i0 < NBLK; i0 += HB) {
+          typename mma<T>::frag vf[2][HB];
+#pragma unroll
+          for (int i = 0; i < HB; ++i) vf[0][i] = mma<T>::load(vp + (i0 + i) * 32 * VROW);
+#pragma unroll
+          for (int st = 0; st < 2 * KB; ++st) {     // k-step st covers keys st*16 .. st*16+15 of the tile
+            if (dbg & 1) break;
+            const int cur = st & 1, nxt = cur ^ 1;
+            if (st + 1 < 2 * KB) {
+#pragma unroll
+              for (int i = 0; i < HB; ++i) vf[nxt][i] = mma<T>::load(vp + (i0 + i) * 32 * VROW + (st + 1) * 16);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < HB; ++i) mma<T>::run(o[i0 + i], vf[cur][i], pf[st / 2][st % 2]);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      }
+    }
+    if (kt + 1 < ntiles && !(dbg & 8)) {
+      store_tile(buf ^ 1);
+      if ((kt + 2) * BKV - 1 > klast) {     // only the last tile of a sequence can be partial
+        __syncthreads();
+        fix_last_tile(kt + 1, buf ^ 1);
       }
     }
     __syncthreads();
-    // wave-uniform skip of tiles that lie entirely above this wavefront's last query
-    const int wave_last = qt0 + wave * 32 + 31 + p0;
-    if (key0 > wave_last) continue;
-
-    // ---- S^T tile: rows = (permuted) keys, columns = queries
-    floatx16 s;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) s[v] = 0.f;
-    {
-      const T* kp = Ks + krow * KROW + fg * 8;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) mma<T>::run(s, mma<T>::load(kp + ks * 16), qf[ks]);
-    }
-    // register v of this lane is key key0 + 16*(v/8) + 8*fg + v%8
-    float p[16];
-    float mt = -INFINITY;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int key = key0 + 16 * (v / 8) + 8 * fg + (v % 8);
-      const bool ok = key <= qpos;
-      p[v] = ok ? s[v] * scale : -INFINITY;
-      mt = fmaxf(mt, p[v]);
-    }
-    mt = fmaxf(mt, __shfl_xor(mt, 32));
-    const float mnew = fmaxf(mrun, mt);
-    const float msafe = (mnew == -INFINITY) ? 0.f : mnew;
-    const float alpha = expf(mrun - msafe);      // mrun = -inf -> 0
-    float lt = 0.f;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      p[v] = expf(p[v] - msafe);                 // masked -> exp(-inf) = 0
-      lt += p[v];
-    }
-    lt += __shfl_xor(lt, 32);
-    lrun = lrun * alpha + lt;
-    mrun = mnew;
-#pragma unroll
-    for (int i = 0; i < NBLK; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
-
-    // ---- O^T += V^T P^T : A = V^T rows (head-dim), B = P^T (keys x queries)
-    const typename mma<T>::frag pf0 = mma<T>::from_floats(p), pf1 = mma<T>::from_floats(p + 8);
-#pragma unroll
-    for (int i = 0; i < NBLK; ++i) {
-      const T* vp = Vs + (i * 32 + fr) * VROW + fg * 8;
-      mma<T>::run(o[i], mma<T>::load(vp), pf0);
-      mma<T>::run(o[i], mma<T>::load(vp + 16), pf1);
-    }
   }
 
   // ---- write O: register v of block i is head-dim i*32 + 8*(v/4) + 4*fg + v%4 of query t
@@ -196,8 +304,15 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__
 #pragma unroll
       for (int v4 = 0; v4 < 4; ++v4) {
         const int e = i * 32 + 8 * v4 + 4 * fg;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) elem<T>::store(op + e + w, o[i][v4 * 4 + w] * inv);
+        if (sizeof(T) == 2) {
+          uint32x2 pk;
+          pk.x = pack_bf16x2(o[i][v4 * 4] * inv, o[i][v4 * 4 + 1] * inv);
+          pk.y = pack_bf16x2(o[i][v4 * 4 + 2] * inv, o[i][v4 * 4 + 3] * inv);
+          *reinterpret_cast<uint32x2*>(op + e) = pk;
+        } else {
+          *reinterpret_cast<floatx4*>(op + e) =
+              floatx4{o[i][v4 * 4] * inv, o[i][v4 * 4 + 1] * inv, o[i][v4 * 4 + 2] * inv, o[i][v4 * 4 + 3] * inv};
+        }
       }
   }
 }
@@ -355,19 +470,31 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
               "mtj_attn_prefill: bad shape B=%lld H=%lld Tp=%lld Tcap=%lld", (long long)B, (long long)H,
               (long long)Tp, (long long)Tcap);
   const int esz = dtype == MTJ_BF16 ? 2 : 4;
-  MTJ_REQUIRE(ldvt >= Tp && (ldvt * esz) % 16 == 0 && (ld_out * esz) % 16 == 0, MTJ_EALIGN,
-              "mtj_attn_prefill: ldvt must be >= Tp and rows 16-byte aligned");
+  MTJ_REQUIRE(ldvt >= (Tp + 63) / 64 * 64 && (ldvt * esz) % 16 == 0 && (ld_out * esz) % 16 == 0, MTJ_EALIGN,
+              "mtj_attn_prefill: ldvt must be >= Tp rounded up to a multiple of 64, rows 16-byte aligned");
   MTJ_REQUIRE(mtj_aligned16(q) && mtj_aligned16(k_cache) && mtj_aligned16(v_t) && mtj_aligned16(out), MTJ_EALIGN,
               "mtj_attn_prefill: pointers must be 16-byte aligned");
-  dim3 grid((unsigned)((Tp + 127) / 128), (unsigned)H, (unsigned)B);
   hipStream_t s = (hipStream_t)stream;
-#define MTJ_PREFILL(T, DH)                                                                                    \
-  attn_prefill_kernel<T, DH><<<grid, 256, 0, s>>>((const T*)q, (const T*)k_cache, (const T*)v_t, pos0, (int)H, \
-                                                  (int)Tp, (int)Tcap, ldvt, (T*)out, ld_out)
-  if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL(bf16_t, 256);
-  else if (dtype == MTJ_BF16 && dh == 64) MTJ_PREFILL(bf16_t, 64);
-  else if (dtype == MTJ_F32 && dh == 256) MTJ_PREFILL(float, 256);
-  else if (dtype == MTJ_F32 && dh == 64) MTJ_PREFILL(float, 64);
+#define MTJ_PREFILL(T, DH, NW, BKV)                                                                                  \
+  do {                                                                                                               \
+    constexpr size_t lds = 2 * ((size_t)BKV * (DH + mma<T>::EPC) + (size_t)DH * (BKV + mma<T>::EPC)) * sizeof(T);    \
+    static_assert(lds <= 160 * 1024, "attention tiles do not fit LDS");                                              \
+    static bool attr_set = false;                                                                                    \
+    if (!attr_set) {                                                                                                 \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<T, DH, NW, BKV>),        \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                      \
+      if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_attn_prefill: hipFuncSetAttribute: %s", hipGetErrorString(e)); \
+      attr_set = true;                                                                                               \
+    }                                                                                                                \
+    dim3 grid((unsigned)((Tp + NW * 32 - 1) / (NW * 32)), (unsigned)H, (unsigned)B);                                 \
+    attn_prefill_kernel<T, DH, NW, BKV><<<grid, NW * 64, lds, s>>>((const T*)q, (const T*)k_cache, (const T*)v_t,    \
+                                                                  pos0, (int)H, (int)Tp, (int)Tcap, ldvt, (T*)out,   \
+                                                                  ld_out, getenv("MTJ_ATTN_DBG") ? atoi(getenv("MTJ_ATTN_DBG")) : 0); \
+  } while (0)
+  if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL(bf16_t, 256, 4, 32);
+  else if (dtype == MTJ_BF16 && dh == 64) MTJ_PREFILL(bf16_t, 64, 8, 64);
+  else if (dtype == MTJ_F32 && dh == 256) MTJ_PREFILL(float, 256, 4, 32);
+  else if (dtype == MTJ_F32 && dh == 64) MTJ_PREFILL(float, 64, 4, 32);
   else return mtj_fail(MTJ_EINVAL, "mtj_attn_prefill: unsupported dtype %d / d_head %lld (64 or 256)", dtype, (long long)dh);
 #undef MTJ_PREFILL
   return mtj_check_launch("mtj_attn_prefill");

@@ -32,14 +32,16 @@ static inline bool mtj_aligned16(const void* p) { return (reinterpret_cast<uintp
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t hi16) { return __uint_as_float(hi16 << 16); }
 __device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
+// gfx950 converts in hardware (v_cvt_pk_bf16_f32, round to nearest even)
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;  // NaN stays NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
+  const __bf16 b = (__bf16)f;
+  return (uint32_t)__builtin_bit_cast(uint16_t, b);
 }
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const bf16x2 r = __builtin_convertvector(f32x2{lo, hi}, bf16x2);
+  return __builtin_bit_cast(uint32_t, r);
 }
 
 template <typename T> struct elem;

@@ -110,7 +110,11 @@ class Session:
         self.sin, self.cos = rotary_tables(max_pos, eng.r, dev)
         # prefill buffers
         M = max(B * Tp_max, 1)
-        self.ldvt = max((Tp_max + 31) // 32 * 32, 32)
+        # row length of the transposed-V scratch: a multiple of 64 elements, but never a multiple of 2 KiB in
+        # bytes - rows a power-of-two apart all land in the same memory channel
+        self.ldvt = max((Tp_max + 63) // 64 * 64, 64)
+        if (self.ldvt * (2 if T == torch.bfloat16 else 4)) % 2048 == 0:
+            self.ldvt += 64
         self.x_pf = torch.empty(M, d, dtype=torch.float32, device=dev)
         self.h_pf = torch.empty(M, d, dtype=T, device=dev)
         self.act_pf = torch.empty(M, d + F, dtype=T, device=dev)

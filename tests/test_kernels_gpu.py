@@ -303,7 +303,7 @@ def test_attn_prefill(L, dt, dh, H, Tp):
     g = torch.Generator().manual_seed(Tp + dh)
     B, Tcap = 2, Tp + 3
     pads = [0, min(5, Tp - 1)]
-    ldvt = (Tp + 31) // 32 * 32
+    ldvt = (Tp + 63) // 64 * 64
     q = torch.randn(B, H, Tp, dh, generator=g).to(TD[dt]).to(DEV)
     kc = torch.zeros(B, H, Tcap, dh, dtype=TD[dt], device=DEV)
     vt = torch.full((B, H, dh, ldvt), float("nan"), dtype=TD[dt], device=DEV)   # unwritten keys must never be read

@@ -1,6 +1,5 @@
 // Attention: MFMA flash-style prefill over a left-padded rectangle, and one-token decode over the K/V window.
 #include "mtj_common.h"
-#include <cstdlib>
 
 namespace {
 
@@ -68,7 +67,7 @@ template <typename T, int DH, int NW, int BKV>
 __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ kc,
                                                                const T* __restrict__ vt, const int32_t* __restrict__ pos0,
                                                                int H, int Tp, int Tcap, int64_t ldvt, T* __restrict__ out,
-                                                               int64_t ld_out, int dbg) {
+                                                               int64_t ld_out) {
   constexpr int NT = NW * 64;
   constexpr int BQ = NW * 32;
   constexpr int EPC = mma<T>::EPC;
@@ -172,7 +171,7 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
   for (int kt = 0; kt < ntiles; ++kt) {
     const int buf = kt & 1;
     const int key0 = kt * BKV;
-    if (kt + 1 < ntiles && !(dbg & 8)) load_tile(kt + 1);
+    if (kt + 1 < ntiles) load_tile(kt + 1);
     if (key0 <= wave_last) {      // wave-uniform: tiles entirely above this wavefront's last query are skipped
       // ---- S^T blocks: rows = (permuted) keys, columns = queries.  The K fragments of k-steps
       // ks+G .. ks+2G-1 are read from LDS while the MFMAs of k-steps ks .. ks+G-1 run; the KB key blocks
@@ -192,7 +191,6 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
           for (int g = 0; g < G; ++g) kf[0][kb][g] = mma<T>::load(kp + kb * 32 * KROW + g * 16);
 #pragma unroll
         for (int k0 = 0; k0 < KS; k0 += G) {
-          if (dbg & 2) break;
           const int cur = (k0 / G) & 1, nxt = cur ^ 1;
           if (k0 + G < KS) {
 #pragma unroll
@@ -210,7 +208,6 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
       }
       // register v of block kb is key key0 + kb*32 + 16*(v/8) + 8*fg + v%8
       float mt = -INFINITY;
-      if (dbg & 4) { mt = s[0][0]; } else
       if (key0 + BKV - 1 <= wave_first) {   // wave-uniform: the whole tile is below the diagonal for every lane
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
@@ -271,7 +268,6 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
           for (int i = 0; i < HB; ++i) vf[0][i] = mma<T>::load(vp + (i0 + i) * 32 * VROW);
 #pragma unroll
           for (int st = 0; st < 2 * KB; ++st) {     // k-step st covers keys st*16 .. st*16+15 of the tile
-            if (dbg & 1) break;
             const int cur = st & 1, nxt = cur ^ 1;
             if (st + 1 < 2 * KB) {
 #pragma unroll
@@ -285,7 +281,7 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
         }
       }
     }
-    if (kt + 1 < ntiles && !(dbg & 8)) {
+    if (kt + 1 < ntiles) {
       store_tile(buf ^ 1);
       if ((kt + 2) * BKV - 1 > klast) {     // only the last tile of a sequence can be partial
         __syncthreads();
@@ -489,7 +485,7 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
     dim3 grid((unsigned)((Tp + NW * 32 - 1) / (NW * 32)), (unsigned)H, (unsigned)B);                                 \
     attn_prefill_kernel<T, DH, NW, BKV><<<grid, NW * 64, lds, s>>>((const T*)q, (const T*)k_cache, (const T*)v_t,    \
                                                                   pos0, (int)H, (int)Tp, (int)Tcap, ldvt, (T*)out,   \
-                                                                  ld_out, getenv("MTJ_ATTN_DBG") ? atoi(getenv("MTJ_ATTN_DBG")) : 0); \
+                                                                  ld_out); \
   } while (0)
   if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL(bf16_t, 256, 4, 32);
   else if (dtype == MTJ_BF16 && dh == 64) MTJ_PREFILL(bf16_t, 64, 8, 64);

@@ -1,7 +1,10 @@
 // MFMA GEMM for prefill and batched decode: C[M, N] = A[M, K] x W[N, K]^T with fused epilogues.
-// Both operands are K-contiguous, are staged global -> registers -> LDS (padded rows, so that the
-// 16-byte fragment reads of a 32x32 MFMA hit distinct banks) and double-buffered; accumulation is
-// float32.  bf16 uses v_mfma_f32_32x32x16_bf16, float32 uses v_mfma_f32_32x32x2_f32 (true fp32).
+// Both operands are K-contiguous and accumulation is float32; bf16 uses v_mfma_f32_32x32x16_bf16, float32 uses
+// v_mfma_f32_32x32x2_f32 (true fp32).  Two kernels share the epilogues:
+//   gemm_kernel      any dtype and shape: global -> registers -> LDS (padded rows, so that the 16-byte fragment
+//                    reads of a 32x32 MFMA hit distinct banks), LDS double-buffered;
+//   gemm_dma_kernel  large bf16 problems: 256x256x64 tiles written straight into LDS by the memory pipeline
+//                    (buffer_load ... lds), rows xor-swizzled instead of padded, no staging registers.
 #include "mtj_common.h"
 #include <type_traits>
 
@@ -88,6 +91,150 @@ template <int S, int NS, class F>
 __device__ __forceinline__ void for_stages(F&& f) {
   f(std::integral_constant<int, S>{});
   if constexpr (S + 1 < NS) for_stages<S + 1, NS>(f);
+}
+
+// per-tile operands of the fused input-projection epilogue, fetched one tile ahead of their use:
+// fc_in columns: 16 bias values; rotary q/k columns: 8 sines then 8 cosines
+struct epi_ops { floatx4 o[4]; };
+
+// Epilogue of a workgroup tile whose wavefront (wm, wn) holds WM x WN accumulator tiles of 32x32; accumulator
+// register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32].  `smem` (the operand staging area, no longer
+// needed) must hold 2*BM ints and one 32x36 float patch per wavefront.
+template <int EPI, int WAVES_M, int WAVES_N, int WM, int WN>
+__device__ __forceinline__ void epilogue(const gemm_args& a, floatx16 (&acc)[WM][WN], unsigned char* smem, int m0, int n0) {
+  constexpr int NT = WAVES_M * WAVES_N * 64, BM = WAVES_M * WM * 32;
+  constexpr int PS = 36;   // patch row stride in floats: 16-byte aligned rows, and 16-byte reads of 8 lanes hit distinct banks
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int fr = lane & 31, fg = lane >> 5;
+  if (EPI == MTJ_EPI_INPROJ) {
+    // Each 32x32 accumulator tile goes through a private LDS patch of its wavefront and comes back with one
+    // lane owning 16 consecutive columns of one row: rotary pairs are then lane-local and every destination
+    // (q, K/V window, gelu(fc_in)) gets 32- or 64-byte stores.
+    __syncthreads();                                       // every wavefront is done with the operand tiles
+    int* row_b = reinterpret_cast<int*>(smem);
+    int* row_pos = row_b + BM;
+    float* patch = reinterpret_cast<float*>(smem) + 2 * BM + wave * (32 * PS);
+    for (int r = tid; r < BM; r += NT) {
+      const int m = m0 + r;
+      int b = 0, pos = -1;
+      if (m < a.M) {
+        b = m / a.ip.Tp;
+        pos = a.ip.pos0[b] + (m - b * a.ip.Tp);
+      }
+      row_b[r] = b;
+      row_pos[r] = pos;
+    }
+    __syncthreads();
+    const int d = a.ip.n_heads * a.ip.d_head, dh = a.ip.d_head, rd = a.ip.rotary_dims, Tp = a.ip.Tp;
+    const int prow = lane >> 1, pcol = (lane & 1) * 16;     // my row / first column inside a tile
+
+    // tile-uniform facts of accumulator tile column j, and my first column inside its segment
+    struct col_info { bool is_fc, n_ok; int seg, c0, h, e0; };
+    auto column = [&](int j) {
+      col_info c;
+      const int nb = n0 + (wn * WN + j) * 32;               // first column of the tile
+      c.is_fc = nb >= 3 * d;
+      c.seg = c.is_fc ? 3 : nb / d;                         // 0 q, 1 v, 2 k
+      c.c0 = nb - c.seg * d + pcol;
+      c.h = c.c0 / dh;
+      c.e0 = c.c0 - c.h * dh;
+      c.n_ok = nb + pcol < a.N;                             // N is a multiple of 16 columns here
+      return c;
+    };
+    auto load_ops = [&](int i, int j) {
+      epi_ops p;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) p.o[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+      const col_info c = column(j);
+      if (!c.n_ok) return p;
+      if (c.is_fc) {
+        const floatx4* bp = reinterpret_cast<const floatx4*>(a.bias + c.c0);   // c0 is a multiple of 16
+#pragma unroll
+        for (int q = 0; q < 4; ++q) p.o[q] = bp[q];
+      } else if (c.seg != 1 && c.e0 < rd) {                 // rd is a multiple of 16 (checked on the host)
+        const int pos = row_pos[(wm * WM + i) * 32 + prow];
+        if (pos >= 0) {
+          const int pp = pos < a.ip.max_pos ? pos : a.ip.max_pos - 1;
+          const floatx4* sp = reinterpret_cast<const floatx4*>(a.ip.sin_tab + (int64_t)pp * (rd / 2) + (c.e0 >> 1));
+          const floatx4* cp = reinterpret_cast<const floatx4*>(a.ip.cos_tab + (int64_t)pp * (rd / 2) + (c.e0 >> 1));
+          p.o[0] = sp[0]; p.o[1] = sp[1]; p.o[2] = cp[0]; p.o[3] = cp[1];
+        }
+      }
+      return p;
+    };
+    epi_ops cur = load_ops(0, 0);
+    for_tiles<0, 0, WM, WN>([&](auto I_, auto J_) {
+      constexpr int i = decltype(I_)::value, j = decltype(J_)::value;
+      constexpr int ni = i + 1 < WM ? i + 1 : 0, nj = i + 1 < WM ? j : j + 1;
+      epi_ops nxt = cur;
+      if constexpr (nj < WN) nxt = load_ops(ni, nj);
+      const col_info c = column(j);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) patch[(8 * (v / 4) + 4 * fg + (v % 4)) * PS + fr] = acc[i][j][v];
+      __builtin_amdgcn_wave_barrier();
+      float val[16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const floatx4 t = *reinterpret_cast<const floatx4*>(patch + prow * PS + pcol + 4 * q);
+        val[4 * q] = t.x; val[4 * q + 1] = t.y; val[4 * q + 2] = t.z; val[4 * q + 3] = t.w;
+      }
+      __builtin_amdgcn_wave_barrier();
+      const int r = (wm * WM + i) * 32 + prow;
+      const int m = m0 + r;
+      if (m < a.M && c.n_ok) {
+        if (c.is_fc) {
+#pragma unroll
+          for (int k = 0; k < 16; ++k) val[k] = gelu_tanh(val[k] + cur.o[k >> 2][k & 3]);
+          store16(a.ip.act, (int64_t)m * a.ip.ld_act + d + c.c0, val, a.ip.act_dtype);
+        } else {
+          const int pos = row_pos[r];
+          if (pos >= 0) {
+            const int b = row_b[r];
+            if (c.seg != 1 && c.e0 < rd) {
+#pragma unroll
+              for (int k = 0; k < 16; k += 2) {
+                const float sn = cur.o[k >> 3][(k >> 1) & 3], cs = cur.o[2 + (k >> 3)][(k >> 1) & 3];
+                const float x0 = val[k], x1 = val[k + 1];
+                val[k] = x0 * cs - x1 * sn;
+                val[k + 1] = x1 * cs + x0 * sn;
+              }
+            }
+            const int64_t bh = (int64_t)b * a.ip.n_heads + c.h;
+            if (c.seg == 0) {
+              store16(a.ip.q, (bh * Tp + (m - b * Tp)) * dh + c.e0, val, a.ip.q_dtype);
+            } else {
+              const int slot = pos % a.ip.Tcap;
+              store16(c.seg == 1 ? a.ip.v_cache : a.ip.k_cache, (bh * a.ip.Tcap + slot) * dh + c.e0, val, a.kv_dtype);
+              if (c.seg == 1 && a.ip.v_t && pos < a.ip.ldvt) {
+#pragma unroll
+                for (int k = 0; k < 16; ++k) store_as(a.ip.v_t, (bh * dh + c.e0 + k) * a.ip.ldvt + pos, val[k], a.kv_dtype);
+              }
+            }
+          }
+        }
+      }
+      cur = nxt;
+    });
+  } else {
+    for_tiles<0, 0, WM, WN>([&](auto I_, auto J_) {
+      constexpr int i = decltype(I_)::value, j = decltype(J_)::value;
+      const int n = n0 + (wn * WN + j) * 32 + fr;
+      const bool n_ok = n < a.N;
+      const float bias = (a.bias && n_ok) ? a.bias[n] : 0.f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + (wm * WM + i) * 32 + 8 * (v / 4) + 4 * fg + (v % 4);
+        if (m < a.M && n_ok) {
+          const int64_t idx = (int64_t)m * a.ldo + n;
+          const float val = acc[i][j][v] + bias;
+          if (EPI == MTJ_EPI_RESID) reinterpret_cast<float*>(a.out)[idx] += val;
+          else if (a.out_dtype == MTJ_F32) reinterpret_cast<float*>(a.out)[idx] = val;
+          else reinterpret_cast<uint16_t*>(a.out)[idx] = (uint16_t)f32_to_bf16_bits(val);
+        }
+      }
+    });
+  }
 }
 
 // Workgroup tile (WAVES_M*WM*32) x (WAVES_N*WN*32), K step BK elements, NS register stages, epilogue EPI.
@@ -191,17 +338,27 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
     const int buf = kt & 1;
     const T* as = As + (buf * BM + wm * WM * 32 + fr) * LDS_ROW + fg * 8;
     const T* bs = Bs + (buf * BN + wn * WN * 32 + fr) * LDS_ROW + fg * 8;
+    // fragments of k-step ks+1 are read from LDS while the MFMAs of k-step ks run
+    typename mma<T>::frag fa[2][WM], fb[2][WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i) fa[0][i] = mma<T>::load(as + i * 32 * LDS_ROW);
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fb[0][j] = mma<T>::load(bs + j * 32 * LDS_ROW);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
-      typename mma<T>::frag fa[WM], fb[WN];
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks + 1 < BK / 16) {
 #pragma unroll
-      for (int i = 0; i < WM; ++i) fa[i] = mma<T>::load(as + i * 32 * LDS_ROW + ks * 16);
+        for (int i = 0; i < WM; ++i) fa[nxt][i] = mma<T>::load(as + i * 32 * LDS_ROW + (ks + 1) * 16);
 #pragma unroll
-      for (int j = 0; j < WN; ++j) fb[j] = mma<T>::load(bs + j * 32 * LDS_ROW + ks * 16);
+        for (int j = 0; j < WN; ++j) fb[nxt][j] = mma<T>::load(bs + j * 32 * LDS_ROW + (ks + 1) * 16);
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < WM; ++i)
 #pragma unroll
-        for (int j = 0; j < WN; ++j) mma<T>::run(acc[i][j], fa[i], fb[j]);
+        for (int j = 0; j < WN; ++j) mma<T>::run(acc[i][j], fa[cur][i], fb[cur][j]);
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (kt + 1 < KT) store_lds(PARK_, buf ^ 1);
     if (kt + 1 + NS < KT) load_global(PARK_, kt + 1 + NS);
@@ -214,101 +371,163 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
     });
   }
 
-  // ---- epilogue.  Accumulator register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32].
-  if (EPI == MTJ_EPI_INPROJ) {
-    // Each 32x32 accumulator tile goes through a private LDS patch of its wavefront and comes back with one
-    // lane owning 16 consecutive columns of one row: rotary pairs are then lane-local and every destination
-    // (q, K/V window, gelu(fc_in)) gets 32- or 64-byte stores.  The operand tiles are no longer needed.
-    int* row_b = reinterpret_cast<int*>(smem);
-    int* row_pos = row_b + BM;
-    float* patch = reinterpret_cast<float*>(smem) + 2 * BM + wave * (32 * 33);
-    for (int r = tid; r < BM; r += NT) {
-      const int m = m0 + r;
-      int b = 0, pos = -1;
-      if (m < a.M) {
-        b = m / a.ip.Tp;
-        pos = a.ip.pos0[b] + (m - b * a.ip.Tp);
-      }
-      row_b[r] = b;
-      row_pos[r] = pos;
-    }
-    __syncthreads();
-    const int d = a.ip.n_heads * a.ip.d_head, dh = a.ip.d_head, rd = a.ip.rotary_dims, Tp = a.ip.Tp;
-    const int prow = lane >> 1, pcol = (lane & 1) * 16;     // my row / first column inside a tile
-    for_tiles<0, 0, WM, WN>([&](auto I_, auto J_) {
-      constexpr int i = decltype(I_)::value, j = decltype(J_)::value;
-      const int nb = n0 + (wn * WN + j) * 32;               // first column of this tile (tile-uniform facts below)
-      const bool is_fc = nb >= 3 * d;
-      const int seg = is_fc ? 3 : nb / d;                   // 0 q, 1 v, 2 k
-      const int c0 = nb - seg * d + pcol;                   // my first column inside the segment
-      const int h = c0 / dh, e0 = c0 - h * dh;
-      const bool n_ok = nb + pcol < a.N;                    // N is a multiple of 16 columns here
-      {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) patch[(8 * (v / 4) + 4 * fg + (v % 4)) * 33 + fr] = acc[i][j][v];
-        __builtin_amdgcn_wave_barrier();
-        float val[16];
-#pragma unroll
-        for (int k = 0; k < 16; ++k) val[k] = patch[prow * 33 + pcol + k];
-        __builtin_amdgcn_wave_barrier();
-        const int r = (wm * WM + i) * 32 + prow;
-        const int m = m0 + r;
-        if (m < a.M && n_ok) {
-          if (is_fc) {
-#pragma unroll
-            for (int k = 0; k < 16; ++k) val[k] = gelu_tanh(val[k] + a.bias[c0 + k]);
-            store16(a.ip.act, (int64_t)m * a.ip.ld_act + d + c0, val, a.ip.act_dtype);
-          } else {
-            const int pos = row_pos[r];
-            if (pos >= 0) {
-              const int b = row_b[r];
-              if (seg != 1 && e0 < rd) {                    // rd is a multiple of 16 (checked on the host)
-                const int pp = pos < a.ip.max_pos ? pos : a.ip.max_pos - 1;
-                const float* sp = a.ip.sin_tab + (int64_t)pp * (rd / 2) + (e0 >> 1);
-                const float* cp = a.ip.cos_tab + (int64_t)pp * (rd / 2) + (e0 >> 1);
-#pragma unroll
-                for (int k = 0; k < 16; k += 2) {
-                  const float sn = sp[k >> 1], cs = cp[k >> 1];
-                  const float x0 = val[k], x1 = val[k + 1];
-                  val[k] = x0 * cs - x1 * sn;
-                  val[k + 1] = x1 * cs + x0 * sn;
-                }
-              }
-              const int64_t bh = (int64_t)b * a.ip.n_heads + h;
-              if (seg == 0) {
-                store16(a.ip.q, (bh * Tp + (m - b * Tp)) * dh + e0, val, a.ip.q_dtype);
-              } else {
-                const int slot = pos % a.ip.Tcap;
-                store16(seg == 1 ? a.ip.v_cache : a.ip.k_cache, (bh * a.ip.Tcap + slot) * dh + e0, val, a.kv_dtype);
-                if (seg == 1 && a.ip.v_t && pos < a.ip.ldvt) {
-#pragma unroll
-                  for (int k = 0; k < 16; ++k) store_as(a.ip.v_t, (bh * dh + e0 + k) * a.ip.ldvt + pos, val[k], a.kv_dtype);
-                }
-              }
-            }
-          }
-        }
-      }
-    });
-  } else {
-    for_tiles<0, 0, WM, WN>([&](auto I_, auto J_) {
-      constexpr int i = decltype(I_)::value, j = decltype(J_)::value;
-      const int n = n0 + (wn * WN + j) * 32 + fr;
-      const bool n_ok = n < a.N;
-      const float bias = (a.bias && n_ok) ? a.bias[n] : 0.f;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m0 + (wm * WM + i) * 32 + 8 * (v / 4) + 4 * fg + (v % 4);
-        if (m < a.M && n_ok) {
-          const int64_t idx = (int64_t)m * a.ldo + n;
-          const float val = acc[i][j][v] + bias;
-          if (EPI == MTJ_EPI_RESID) reinterpret_cast<float*>(a.out)[idx] += val;
-          else if (a.out_dtype == MTJ_F32) reinterpret_cast<float*>(a.out)[idx] = val;
-          else reinterpret_cast<uint16_t*>(a.out)[idx] = (uint16_t)f32_to_bf16_bits(val);
-        }
-      }
-    });
+  epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, acc, smem, m0, n0);
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+// s_waitcnt immediates that constrain one counter only (gfx9 encoding: vmcnt [3:0] and [15:14], expcnt [6:4],
+// lgkmcnt [11:8])
+constexpr int wait_vmcnt(int n) { return (n & 0xf) | (((n >> 4) & 3) << 14) | (0x7 << 4) | (0xf << 8); }
+constexpr int wait_lgkmcnt(int n) { return 0xf | (3 << 14) | (0x7 << 4) | ((n & 0xf) << 8); }
+
+// bf16, 256x256 workgroup tile, 8 wavefronts of 128x64, K step 64, two LDS stages of 64 KiB.
+//
+// The memory pipeline writes the operand tiles straight into LDS (buffer_load_dwordx4 ... lds: 64 lanes x
+// 16 bytes land at consecutive LDS addresses), so there are no staging registers, no ds_write and the loads
+// of k-tile kt+2 are in flight while k-tile kt+1 waits in LDS.  A tile row is 128 bytes = 8 chunks; LDS
+// position (row, c) holds chunk c ^ ((row >> 1) & 7) of the row, which each lane arranges by choosing its
+// global address, and which makes the 16-byte fragment reads of 16 consecutive rows hit 16 distinct bank
+// groups without padding.  One barrier per k-tile, placed before the last of the four MFMA steps: behind it
+// k-tile kt+1 is visible to everyone and k-tile kt has been read by everyone, so the first fragments of kt+1
+// are fetched under the last MFMAs of kt and the stage of kt is handed to the loads of kt+2.  Those eight
+// loads per wavefront are issued one per two MFMAs (a burst would stall the wavefront on the address queue
+// with its MFMAs behind it).  Rows beyond M or N are outside the buffer resource and read as zero.
+template <int EPI>
+__global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
+  using T = bf16_t;
+  constexpr int WAVES_M = 2, WAVES_N = 4, WM = 4, WN = 2, NT = 512, BM = 256, BN = 256, BK = 64, NST = 2;
+  constexpr int ROWB = BK * 2, CPR = BK / 8, OPB = BM * ROWB, STAGEB = 2 * OPB;
+  constexpr int LOADS = BM * CPR / NT, ROWS_PER_LOAD = NT / CPR, KS = BK / 16;
+  static_assert(WM * WN == 2 * LOADS, "one load per two MFMAs");
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int fr = lane & 31, fg = lane >> 5;
+
+  // tile id: as in gemm_kernel (contiguous tile ranges per XCD, groups of 8 row-tiles)
+  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+  const int nblk = tiles_m * tiles_n;
+  int pid = blockIdx.x;
+  {
+    const int per = nblk / 8;
+    if (pid < per * 8) pid = (pid % 8) * per + pid / 8;
   }
+  constexpr int GM = 8;
+  const int group = pid / (GM * tiles_n);
+  const int first_m = group * GM;
+  const int gsz = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;
+  const int tm = first_m + (pid % (GM * tiles_n)) % gsz;
+  const int tn = (pid % (GM * tiles_n)) / gsz;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int rows_a = (a.M - m0 < BM) ? a.M - m0 : BM, rows_b = (a.N - n0 < BN) ? a.N - n0 : BN;
+  const T* tile_a = reinterpret_cast<const T*>(a.A) + (int64_t)m0 * a.lda;
+  const T* tile_b = reinterpret_cast<const T*>(a.W) + (int64_t)n0 * a.K;
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(tile_a), 0, (int)((((int64_t)rows_a - 1) * a.lda + a.K) * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(tile_b), 0, (int)((((int64_t)rows_b - 1) * a.K + a.K) * 2), 0x00020000);
+  auto swz = [](int row) { return (row >> 1) & 7; };
+  const int lr = tid / CPR;                                  // my row inside one load's 64 rows
+  const int lc = ((tid % CPR) ^ swz(lr)) * 16;               // byte offset of the chunk I fetch for my LDS position
+  const int voff_a = (int)((int64_t)lr * a.lda * 2) + lc, voff_b = (int)((int64_t)lr * a.K * 2) + lc;
+  const int pass_a = (int)((int64_t)ROWS_PER_LOAD * a.lda * 2), pass_b = (int)((int64_t)ROWS_PER_LOAD * a.K * 2);
+
+  // load number l of a k-tile: l < LOADS fetches rows [l*64, l*64+64) of A, the others of W
+  auto issue_one = [&](int st, int kt, auto L_) {
+    constexpr int l = decltype(L_)::value, part = l / LOADS, i = l % LOADS;
+    unsigned char* dst = smem + st * STAGEB + part * OPB + i * (NT * 16) + wave_s * 1024;
+    if (part == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr)dst, 16, voff_a, kt * ROWB + i * pass_a, 0, 0);
+    else __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr)dst, 16, voff_b, kt * ROWB + i * pass_b, 0, 0);
+  };
+
+  floatx16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int KT = a.K / BK;
+  for_stages<0, 2 * LOADS>([&](auto L_) { issue_one(0, 0, L_); });
+  if (KT > 1) for_stages<0, 2 * LOADS>([&](auto L_) { issue_one(1, 1, L_); });
+
+  // fragment addresses: lane (fr, fg) reads chunk (2*ks + fg) ^ swz(fr) of its row in k-step ks
+  int xo[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) xo[ks] = ((2 * ks + fg) ^ swz(fr)) * 16;
+  const int a_row = (wm * WM * 32 + fr) * ROWB, b_row = OPB + (wn * WN * 32 + fr) * ROWB;
+  bf16x8 fa[2][WM], fb[2][WN];
+  auto read_frags = [&](int st, int ks, int slot) {
+    const unsigned char* p = smem + st * STAGEB + xo[ks];
+#pragma unroll
+    for (int i = 0; i < WM; ++i) fa[slot][i] = *reinterpret_cast<const bf16x8*>(p + a_row + i * 32 * ROWB);
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fb[slot][j] = *reinterpret_cast<const bf16x8*>(p + b_row + j * 32 * ROWB);
+  };
+  if (KT > 1) __builtin_amdgcn_s_waitcnt(wait_vmcnt(2 * LOADS));
+  else __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
+  __builtin_amdgcn_s_barrier();
+  read_frags(0, 0, 0);
+
+  auto k_tile = [&](int kt, auto ST_) {
+    constexpr int st = decltype(ST_)::value;
+    for_stages<0, KS>([&](auto KS_) {
+      constexpr int ks = decltype(KS_)::value, cur = ks & 1, nxt = cur ^ 1;
+      // loads of k-tile kt+2 go out behind the barrier of k-tile kt: the first half under the last step of kt,
+      // the second half under the first step of kt+1 (where they are the loads "of" kt-1+2)
+      constexpr bool first_half = ks == KS - 1, second_half = ks == 0;
+      constexpr int l_st = first_half ? st : st ^ 1;
+      const int l_kt = first_half ? kt + NST : kt - 1 + NST;
+      const bool go = first_half ? (kt + NST < KT) : (kt >= 1 && kt - 1 + NST < KT);
+      if constexpr (ks + 1 < KS) {
+        read_frags(st, ks + 1, nxt);
+      } else {
+        if (kt + 1 < KT) {
+          __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));       // my part of k-tile kt+1 has landed
+          __builtin_amdgcn_s_waitcnt(wait_lgkmcnt(0));     // my fragment reads of k-tile kt have landed
+          __builtin_amdgcn_s_barrier();
+          read_frags(st ^ 1, 0, nxt);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      for_stages<0, WM * WN>([&](auto Q_) {
+        constexpr int q = decltype(Q_)::value, i = q / WN, j = q % WN;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+        if constexpr ((first_half || second_half) && (q & 1)) {
+          __builtin_amdgcn_sched_barrier(0);
+          if (go) issue_one(l_st, l_kt, std::integral_constant<int, (first_half ? 0 : LOADS) + q / 2>{});
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  for (int kt = 0; kt < KT; kt += NST)
+    for_stages<0, NST>([&](auto S_) {
+      if (kt + decltype(S_)::value < KT) k_tile(kt + decltype(S_)::value, S_);
+    });
+
+  epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, acc, smem, m0, n0);
+}
+
+template <int EPI>
+int launch_dma(const gemm_args& a, hipStream_t s) {
+  constexpr size_t lds = 2 * 2 * 256 * 64 * 2;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<EPI>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_gemm: hipFuncSetAttribute: %s", hipGetErrorString(e));
+    attr_set = true;
+  }
+  const int tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
+  gemm_dma_kernel<EPI><<<tiles, 512, lds, s>>>(a);
+  return mtj_check_launch("mtj_gemm");
 }
 
 template <typename T, int EPI, int WAVES_M, int WAVES_N, int WM, int WN, int BK, int NS>
@@ -316,7 +535,7 @@ int launch(const gemm_args& a, hipStream_t s) {
   constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
   constexpr size_t lds = 2 * (size_t)(BM + BN) * (BK + mma<T>::EPC) * sizeof(T);
   static_assert(lds <= 160 * 1024, "tile does not fit LDS");
-  static_assert(lds >= 2 * BM * sizeof(int) + WAVES_M * WAVES_N * 32 * 33 * sizeof(float), "epilogue scratch does not fit");
+  static_assert(lds >= 2 * BM * sizeof(int) + WAVES_M * WAVES_N * 32 * 36 * sizeof(float), "epilogue scratch does not fit");
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK, NS>),
@@ -333,8 +552,10 @@ template <typename T, int EPI, int BK>
 int dispatch_tile(const gemm_args& a, hipStream_t s) {
   if (a.M <= 32) return launch<T, EPI, 1, 4, 1, 2, BK, 2>(a, s);    // 32 x 256: batched decode, weights stream once
   if (a.M <= 64) return launch<T, EPI, 1, 4, 2, 2, BK, 2>(a, s);    // 64 x 256
-  const int64_t big = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
-  if (big >= 200) return launch<T, EPI, 2, 4, 4, 2, BK, 2>(a, s);   // 256 x 256, 8 wavefronts of 128 x 64
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    const int64_t big = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
+    if (big >= 200) return launch_dma<EPI>(a, s);                   // 256 x 256, 8 wavefronts of 128 x 64
+  }
   return launch<T, EPI, 2, 2, 2, 2, BK, 2>(a, s);                   // 128 x 128
 }
 
@@ -376,6 +597,8 @@ extern "C" int mtj_gemm(const void* A, int64_t lda, const void* W, const float* 
                     (ip->act_dtype == MTJ_F32 || ip->act_dtype == MTJ_BF16) &&
                     (ip->q_dtype == MTJ_F32 || ip->q_dtype == MTJ_BF16) && (!ip->v_t || ip->ldvt >= ip->Tp),
                 MTJ_EINVAL, "mtj_gemm: inconsistent INPROJ geometry");
+    MTJ_REQUIRE(mtj_aligned16(bias) && mtj_aligned16(ip->sin_tab) && mtj_aligned16(ip->cos_tab), MTJ_EALIGN,
+                "mtj_gemm: the fc_in bias and the rotary tables must be 16-byte aligned");
   } else if (epi == MTJ_EPI_STORE) {
     MTJ_REQUIRE(out && ldo >= N && (out_dtype == MTJ_F32 || out_dtype == MTJ_BF16), MTJ_EINVAL,
                 "mtj_gemm: STORE needs out with ldo >= N");

@@ -100,6 +100,17 @@ int mtj_layernorm(const float* x, const float* scale, const float* offset, int64
 int mtj_gemm(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
              int dtype, int epi, void* out, int64_t ldo, int out_dtype, const mtj_inproj* ip, void* stream);
 
+/* mtj_gemm for skinny problems (M <= 64: batched decode): when the output has too few tiles to occupy the
+ * chip, K is cut into ranges that run as separate workgroups, each storing a float32 partial tile into `work`,
+ * and a second kernel adds the partials in a fixed order (results do not depend on scheduling) and applies the
+ * epilogue.  STORE and RESID only.  `work` holds mtj_gemm_splitk_work_bytes() bytes (0: no split is used and the
+ * call is mtj_gemm); out and bias must then be 16-byte aligned and ldo a multiple of 4.
+ * Call sites: the out/fc_out projection of decode_once (layers.py:316-344) at batch > 1. */
+int64_t mtj_gemm_splitk_work_bytes(int64_t M, int64_t N, int64_t K, int dtype);
+int mtj_gemm_splitk(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
+                    int dtype, int epi, void* out, int64_t ldo, int out_dtype, void* work, int64_t work_bytes,
+                    void* stream);
+
 /* Batch-1 decode matrix-vector product: y = f(x) @ W^T with float32 activations and float32 accumulation
  * (jnp.dot(f32, bf16) semantics of hk.Linear at decode, layers.py:316-344).  x float32 [K].
  * If ln_scale != NULL the kernel first applies LayerNorm(x) (layers.py:17-36) - x then has K = d entries.

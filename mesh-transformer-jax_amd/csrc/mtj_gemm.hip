@@ -54,6 +54,8 @@ struct gemm_args {
   int64_t ldo;
   int out_dtype;
   int kv_dtype;
+  int splits;             // > 1: blockIdx.y owns a K range and stores a raw float32 partial at out + y * split_stride
+  int64_t split_stride;
   mtj_inproj ip;
 };
 
@@ -101,7 +103,8 @@ struct epi_ops { floatx4 o[4]; };
 // register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32].  `smem` (the operand staging area, no longer
 // needed) must hold 2*BM ints and one 32x36 float patch per wavefront.
 template <int EPI, int WAVES_M, int WAVES_N, int WM, int WN>
-__device__ __forceinline__ void epilogue(const gemm_args& a, floatx16 (&acc)[WM][WN], unsigned char* smem, int m0, int n0) {
+__device__ __forceinline__ void epilogue(const gemm_args& a, void* out, floatx16 (&acc)[WM][WN], unsigned char* smem, int m0,
+                                         int n0) {
   constexpr int NT = WAVES_M * WAVES_N * 64, BM = WAVES_M * WM * 32;
   constexpr int PS = 36;   // patch row stride in floats: 16-byte aligned rows, and 16-byte reads of 8 lanes hit distinct banks
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -228,9 +231,9 @@ __device__ __forceinline__ void epilogue(const gemm_args& a, floatx16 (&acc)[WM]
         if (m < a.M && n_ok) {
           const int64_t idx = (int64_t)m * a.ldo + n;
           const float val = acc[i][j][v] + bias;
-          if (EPI == MTJ_EPI_RESID) reinterpret_cast<float*>(a.out)[idx] += val;
-          else if (a.out_dtype == MTJ_F32) reinterpret_cast<float*>(a.out)[idx] = val;
-          else reinterpret_cast<uint16_t*>(a.out)[idx] = (uint16_t)f32_to_bf16_bits(val);
+          if (EPI == MTJ_EPI_RESID) reinterpret_cast<float*>(out)[idx] += val;
+          else if (a.out_dtype == MTJ_F32) reinterpret_cast<float*>(out)[idx] = val;
+          else reinterpret_cast<uint16_t*>(out)[idx] = (uint16_t)f32_to_bf16_bits(val);
         }
       }
     });
@@ -294,10 +297,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
   const int voff_b = (int)(((int64_t)row0 * a.K + cc0 * EPC) * ESZ);
   const int pass_a = (int)((int64_t)ROWS_PER_PASS * a.lda * ESZ), pass_b = (int)((int64_t)ROWS_PER_PASS * a.K * ESZ);
 
+  const int kt0 = (int)((int64_t)blockIdx.y * (a.K / BK) / a.splits);   // first k-tile of my K range
   uint32x4 ra[NS][A_CHUNKS], rb[NS][B_CHUNKS];
   auto load_global = [&](auto ST_, int kt) {
     constexpr int st = decltype(ST_)::value;
-    const int koff = kt * BK * ESZ;
+    const int koff = (kt0 + kt) * BK * ESZ;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i)
       ra[st][i] = __builtin_amdgcn_raw_buffer_load_b128(ra_rsrc, voff_a, koff + i * pass_a, 0);
@@ -323,7 +327,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  const int KT = a.K / BK;
+  const int KT = (int)((int64_t)(blockIdx.y + 1) * (a.K / BK) / a.splits) - kt0;
   // k-tile t lives in register stage t % NS.  Prologue: request k-tiles 0 .. NS-1, park k-tile 0 in LDS,
   // reuse its stage for k-tile NS.
   for_stages<0, NS>([&](auto ST_) {
@@ -371,7 +375,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
     });
   }
 
-  epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, acc, smem, m0, n0);
+  void* out = a.splits > 1 ? (void*)(reinterpret_cast<float*>(a.out) + blockIdx.y * a.split_stride) : a.out;
+  epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, out, acc, smem, m0, n0);
 }
 
 typedef __attribute__((address_space(3))) void* lds_ptr;
@@ -512,7 +517,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
       if (kt + decltype(S_)::value < KT) k_tile(kt + decltype(S_)::value, S_);
     });
 
-  epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, acc, smem, m0, n0);
+  epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, a.out, acc, smem, m0, n0);
 }
 
 template <int EPI>
@@ -544,7 +549,7 @@ int launch(const gemm_args& a, hipStream_t s) {
     attr_set = true;
   }
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK, NS><<<tiles, WAVES_M * WAVES_N * 64, lds, s>>>(a);
+  gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK, NS><<<dim3(tiles, a.splits), WAVES_M * WAVES_N * 64, lds, s>>>(a);
   return mtj_check_launch("mtj_gemm");
 }
 
@@ -566,26 +571,73 @@ int dispatch(const gemm_args& a, int epi, hipStream_t s) {
   return dispatch_tile<T, MTJ_EPI_INPROJ, BK>(a, s);
 }
 
+// sums the per-split partial tiles in a fixed order and applies the epilogue (four columns per thread)
+template <int EPI>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ work, int splits, int64_t split_stride,
+                                                            int M, int N, const float* __restrict__ bias, void* out,
+                                                            int64_t ldo, int out_dtype) {
+  const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;     // quad index over [M, N / 4]
+  const int nq = N / 4;
+  if (q >= (int64_t)M * nq) return;
+  const int m = (int)(q / nq), n = (int)(q - (int64_t)m * nq) * 4;
+  floatx4 acc = *reinterpret_cast<const floatx4*>(work + (int64_t)m * N + n);
+  for (int sp = 1; sp < splits; ++sp) {
+    const floatx4 p = *reinterpret_cast<const floatx4*>(work + sp * split_stride + (int64_t)m * N + n);
+    acc.x += p.x; acc.y += p.y; acc.z += p.z; acc.w += p.w;
+  }
+  if (bias) {
+    const floatx4 b = *reinterpret_cast<const floatx4*>(bias + n);
+    acc.x += b.x; acc.y += b.y; acc.z += b.z; acc.w += b.w;
+  }
+  const int64_t idx = (int64_t)m * ldo + n;
+  if (EPI == MTJ_EPI_RESID) {
+    float* o = reinterpret_cast<float*>(out) + idx;
+    o[0] += acc.x; o[1] += acc.y; o[2] += acc.z; o[3] += acc.w;
+  } else if (out_dtype == MTJ_F32) {
+    float* o = reinterpret_cast<float*>(out) + idx;
+    o[0] = acc.x; o[1] = acc.y; o[2] = acc.z; o[3] = acc.w;
+  } else {
+    uint16_t* o = reinterpret_cast<uint16_t*>(out) + idx;
+    o[0] = (uint16_t)f32_to_bf16_bits(acc.x); o[1] = (uint16_t)f32_to_bf16_bits(acc.y);
+    o[2] = (uint16_t)f32_to_bf16_bits(acc.z); o[3] = (uint16_t)f32_to_bf16_bits(acc.w);
+  }
+}
+
+// how many K ranges a skinny problem is cut into so that its few output tiles still fill the chip
+int pick_splits(int64_t M, int64_t N, int64_t K, int dtype) {
+  if (M > 64 || N % 4) return 1;
+  const int bk = dtype == MTJ_BF16 ? 64 : 32;
+  const int64_t tiles = (N + 255) / 256, kt = K / bk;
+  int splits = 1;
+  while (splits < 16 && tiles * splits * 2 <= 256 && kt % (splits * 2) == 0 && kt / (splits * 2) >= 4) splits *= 2;
+  return splits;
+}
+
+int check_common(const void* A, int64_t lda, const void* W, int64_t M, int64_t N, int64_t K, int dtype, const char* who) {
+  MTJ_REQUIRE(A && W, MTJ_EINVAL, "%s: null pointer", who);
+  MTJ_REQUIRE(dtype == MTJ_F32 || dtype == MTJ_BF16, MTJ_EDTYPE, "%s: dtype %d", who, dtype);
+  const int bk = dtype == MTJ_BF16 ? 64 : 32;
+  const int esz = dtype == MTJ_BF16 ? 2 : 4;
+  MTJ_REQUIRE(M > 0 && N > 0 && K > 0 && K % bk == 0 && lda >= K, MTJ_EINVAL,
+              "%s: bad shape M=%lld N=%lld K=%lld lda=%lld (K must be a multiple of %d)", who, (long long)M,
+              (long long)N, (long long)K, (long long)lda, bk);
+  MTJ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), MTJ_ELIMIT, "%s: dimension too large", who);
+  MTJ_REQUIRE(mtj_aligned16(A) && mtj_aligned16(W) && (lda * esz) % 16 == 0, MTJ_EALIGN,
+              "%s: A, W and the row stride of A must be 16-byte aligned", who);
+  MTJ_REQUIRE(256 * lda * esz < (1ll << 31) && 256 * K * esz < (1ll << 31), MTJ_ELIMIT,
+              "%s: a 256-row tile of A or W must span less than 2 GiB", who);
+  return MTJ_OK;
+}
+
 }  // namespace
 
 extern "C" int mtj_gemm(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
                         int dtype, int epi, void* out, int64_t ldo, int out_dtype, const mtj_inproj* ip,
                         void* stream) {
-  MTJ_REQUIRE(A && W, MTJ_EINVAL, "mtj_gemm: null pointer");
-  MTJ_REQUIRE(dtype == MTJ_F32 || dtype == MTJ_BF16, MTJ_EDTYPE, "mtj_gemm: dtype %d", dtype);
-  const int bk = dtype == MTJ_BF16 ? 64 : 32;
-  const int esz = dtype == MTJ_BF16 ? 2 : 4;
-  MTJ_REQUIRE(M > 0 && N > 0 && K > 0 && K % bk == 0 && lda >= K, MTJ_EINVAL,
-              "mtj_gemm: bad shape M=%lld N=%lld K=%lld lda=%lld (K must be a multiple of %d)", (long long)M,
-              (long long)N, (long long)K, (long long)lda, bk);
-  MTJ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), MTJ_ELIMIT, "mtj_gemm: dimension too large");
-  MTJ_REQUIRE(mtj_aligned16(A) && mtj_aligned16(W) && (lda * esz) % 16 == 0, MTJ_EALIGN,
-              "mtj_gemm: A, W and the row stride of A must be 16-byte aligned");
-  MTJ_REQUIRE(256 * lda * esz < (1ll << 31) && 256 * K * esz < (1ll << 31), MTJ_ELIMIT,
-              "mtj_gemm: a 256-row tile of A or W must span less than 2 GiB");
+  if (int rc = check_common(A, lda, W, M, N, K, dtype, "mtj_gemm")) return rc;
   gemm_args a{};
   a.A = A; a.lda = lda; a.W = W; a.bias = bias; a.M = (int)M; a.N = (int)N; a.K = (int)K;
-  a.out = out; a.ldo = ldo; a.out_dtype = out_dtype; a.kv_dtype = dtype;
+  a.out = out; a.ldo = ldo; a.out_dtype = out_dtype; a.kv_dtype = dtype; a.splits = 1;
   if (epi == MTJ_EPI_INPROJ) {
     MTJ_REQUIRE(ip && bias, MTJ_EINVAL, "mtj_gemm: INPROJ needs ip and the fc_in bias");
     a.ip = *ip;
@@ -609,4 +661,39 @@ extern "C" int mtj_gemm(const void* A, int64_t lda, const void* W, const float* 
   }
   hipStream_t s = (hipStream_t)stream;
   return dtype == MTJ_BF16 ? dispatch<bf16_t, 64>(a, epi, s) : dispatch<float, 32>(a, epi, s);
+}
+
+extern "C" int64_t mtj_gemm_splitk_work_bytes(int64_t M, int64_t N, int64_t K, int dtype) {
+  if (M <= 0 || N <= 0 || K <= 0 || (dtype != MTJ_F32 && dtype != MTJ_BF16)) return 0;
+  const int splits = pick_splits(M, N, K, dtype);
+  return splits > 1 ? (int64_t)splits * M * N * (int64_t)sizeof(float) : 0;
+}
+
+extern "C" int mtj_gemm_splitk(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N,
+                               int64_t K, int dtype, int epi, void* out, int64_t ldo, int out_dtype, void* work,
+                               int64_t work_bytes, void* stream) {
+  MTJ_REQUIRE(epi == MTJ_EPI_STORE || epi == MTJ_EPI_RESID, MTJ_EINVAL, "mtj_gemm_splitk: epilogue %d", epi);
+  if (int rc = check_common(A, lda, W, M, N, K, dtype, "mtj_gemm_splitk")) return rc;
+  const int splits = pick_splits(M, N, K, dtype);
+  if (splits == 1) return mtj_gemm(A, lda, W, bias, M, N, K, dtype, epi, out, ldo, out_dtype, nullptr, stream);
+  MTJ_REQUIRE(out && ldo >= N && ldo % 4 == 0 && mtj_aligned16(out) && (!bias || mtj_aligned16(bias)), MTJ_EINVAL,
+              "mtj_gemm_splitk: out needs ldo >= N, a multiple of 4, and 16-byte alignment (bias too)");
+  MTJ_REQUIRE(epi == MTJ_EPI_RESID || out_dtype == MTJ_F32 || out_dtype == MTJ_BF16, MTJ_EDTYPE,
+              "mtj_gemm_splitk: out_dtype %d", out_dtype);
+  MTJ_REQUIRE(work && mtj_aligned16(work) && work_bytes >= (int64_t)splits * M * N * (int64_t)sizeof(float), MTJ_EINVAL,
+              "mtj_gemm_splitk: work must hold mtj_gemm_splitk_work_bytes() bytes");
+  gemm_args a{};
+  a.A = A; a.lda = lda; a.W = W; a.bias = nullptr; a.M = (int)M; a.N = (int)N; a.K = (int)K;
+  a.out = work; a.ldo = N; a.out_dtype = MTJ_F32; a.kv_dtype = dtype;
+  a.splits = splits; a.split_stride = M * N;
+  hipStream_t s = (hipStream_t)stream;
+  const int rc = dtype == MTJ_BF16 ? dispatch<bf16_t, 64>(a, MTJ_EPI_STORE, s) : dispatch<float, 32>(a, MTJ_EPI_STORE, s);
+  if (rc) return rc;
+  const int64_t quads = M * (N / 4);
+  const unsigned grid = (unsigned)((quads + 255) / 256);
+  if (epi == MTJ_EPI_RESID)
+    splitk_reduce_kernel<MTJ_EPI_RESID><<<grid, 256, 0, s>>>((const float*)work, splits, M * N, (int)M, (int)N, bias, out, ldo, MTJ_F32);
+  else
+    splitk_reduce_kernel<MTJ_EPI_STORE><<<grid, 256, 0, s>>>((const float*)work, splits, M * N, (int)M, (int)N, bias, out, ldo, out_dtype);
+  return mtj_check_launch("mtj_gemm_splitk");
 }

@@ -128,6 +128,8 @@ class Session:
         self.act = torch.zeros(B, d + F, dtype=act_t, device=dev)
         self.q = torch.empty(B, H, dh, dtype=torch.float32, device=dev)
         self.logits = torch.empty(B, V, dtype=torch.float32, device=dev)
+        nb = 0 if self.gemv_path else L.mtj_gemm_splitk_work_bytes(B, d, d + F, w.dtype)
+        self.gemm_work = torch.empty(max(nb, 256), dtype=torch.uint8, device=dev)
         self.attn_work = torch.zeros(max(L.mtj_attn_decode_work_bytes(B, H, dh, Tcap), 256), dtype=torch.uint8, device=dev)
         self.sample_work = None
         self.tok = torch.zeros(B, dtype=torch.int32, device=dev)
@@ -243,8 +245,8 @@ class Engine:
                              None, 0, 0, C.byref(ip), s))
             check(L.mtj_attn_decode(ptr(ses.q), ptr(ses.kc[i]), ptr(ses.vc[i]), ptr(ses.pos), B, self.H, ses.Tcap,
                                     self.dh, ptr(ses.act), d + F, w.dtype, w.dtype, ptr(ses.attn_work), s))
-            check(L.mtj_gemm(ptr(ses.act), d + F, ptr(w.w_out[i]), ptr(w.b2[i]), B, d, d + F, w.dtype, EPI_RESID,
-                             ptr(ses.x), d, F32, None, s))
+            check(L.mtj_gemm_splitk(ptr(ses.act), d + F, ptr(w.w_out[i]), ptr(w.b2[i]), B, d, d + F, w.dtype, EPI_RESID,
+                                    ptr(ses.x), d, F32, ptr(ses.gemm_work), ses.gemm_work.numel(), s))
 
     def sample_greedy(self, ses, out_tokens, embed_next=True):
         check(_abi.lib().mtj_sample_greedy(ptr(ses.logits), ses.B, self.w.V, ptr(ses.tok), ptr(out_tokens),

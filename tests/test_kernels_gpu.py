@@ -148,6 +148,43 @@ def test_gemm_store_and_resid(L, dt, M, N, K):
     assert rel_err(ob, A.double() @ Wh.double()) < 3e-3
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(32, 4096, 20480), (5, 512, 2560), (64, 260, 1024), (8, 50400, 4096), (3, 64, 64)])
+def test_gemm_splitk_matches_reference_and_is_deterministic(L, dt, M, N, K):
+    """Skinny products: K ranges run as separate workgroups and are added in a fixed order."""
+    a = abi()
+    g = torch.Generator().manual_seed(M * 11 + N)
+    A = torch.randn(M, K, generator=g).to(TD[dt]).to(DEV)
+    Wh = (torch.randn(K, N, generator=g) * 0.05).to(TD[dt]).to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    W = _packed(Wh)
+    ref = A.double() @ Wh.double() + bias.double()
+    code = a.dtype_code(TD[dt])
+    nb = L.mtj_gemm_splitk_work_bytes(M, N, K, code)
+    if (M, N, K) == (32, 4096, 20480):
+        assert nb == 16 * M * N * 4                      # the out/fc_out projection of batched decode is cut 16 ways
+    work = torch.empty(max(nb, 16), dtype=torch.uint8, device=DEV)
+    outs = []
+    for _ in range(2):
+        out = torch.empty(M, N, device=DEV)
+        a.check(L.mtj_gemm_splitk(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_STORE, a.ptr(out), N, 0,
+                                  a.ptr(work), work.numel(), S()))
+        torch.cuda.synchronize()
+        outs.append(out)
+    assert rel_err(outs[0], ref) < 5e-6
+    assert torch.equal(outs[0], outs[1])
+    x0 = torch.randn(M, N, generator=g).to(DEV)
+    x = x0.clone()
+    a.check(L.mtj_gemm_splitk(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_RESID, a.ptr(x), N, 0,
+                              a.ptr(work), work.numel(), S()))
+    torch.cuda.synchronize()
+    assert rel_err(x, x0.double() + ref) < 5e-6
+    if nb:
+        with pytest.raises(ValueError):                  # a work buffer that is too small is refused
+            a.check(L.mtj_gemm_splitk(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_STORE, a.ptr(out), N, 0,
+                                      a.ptr(work), nb - 4, S()))
+
+
 def test_gemm_rejects_bad_arguments(L):
     a = abi()
     A = torch.zeros(4, 48, device=DEV)

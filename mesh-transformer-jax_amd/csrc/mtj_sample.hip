@@ -1,7 +1,7 @@
 // Samplers: greedy argmax, and nucleus (top-k / top-p) filtering with an inverse-CDF draw.
 #include <cstring>
 #include "mtj_common.h"
-#include <rocprim/device/device_segmented_radix_sort.hpp>
+#include <rocprim/device/device_merge_sort.hpp>
 
 namespace {
 
@@ -82,15 +82,19 @@ __device__ __forceinline__ float key_value(uint64_t k) {
   return __uint_as_float(u);
 }
 
-__global__ void make_keys_kernel(const float* __restrict__ logits, int64_t total, int V, uint64_t* __restrict__ keys) {
+// All rows are sorted by one device-wide sort (a sort per row would leave most of the chip idle): bits 48..62
+// carry B-1-row, so that descending order keeps row 0 first and row b occupies [b*V, (b+1)*V) of the output.
+__global__ void make_keys_kernel(const float* __restrict__ logits, int64_t total, int V, int B, uint64_t* __restrict__ keys) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < total) keys[i] = sort_key(logits[i], (uint32_t)(i % V));
+  if (i < total) {
+    const int64_t row = i / V;
+    keys[i] = ((uint64_t)(B - 1 - row) << 48) | sort_key(logits[i], (uint32_t)(i - row * V));
+  }
 }
 
-__global__ void offsets_kernel(uint32_t* off, int B, int V) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i <= B) off[i] = (uint32_t)i * (uint32_t)V;
-}
+struct key_desc {
+  __device__ __forceinline__ bool operator()(const uint64_t& a, const uint64_t& b) const { return a > b; }
+};
 
 // f - a*b with the product rounded to float32 first (no fused multiply-add): logits -= 1e10 * mask is
 // two array operations in the reference (sampling.py:24-26)
@@ -140,7 +144,21 @@ __device__ double block_exclusive(double v, double* sh) {
   return base + inc - v;
 }
 
-// One workgroup per row, each thread owns a contiguous run of the sorted order.
+// wave-wide inclusive prefix sum (double), lanes in order
+__device__ __forceinline__ double wave_inclusive(double v) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const double t = __shfl_up(v, o);
+    if (lane >= o) v += t;
+  }
+  return v;
+}
+
+// One workgroup of 16 wavefronts per row.  Wavefront w owns ranks [w*NT*64, (w+1)*NT*64) of the sorted order in
+// NT tiles of 64 consecutive ranks (lane = rank inside the tile: coalesced reads); the sorted values and ids
+// stay in registers for all three sweeps, and running sums are carried tile to tile inside the wavefront.
+template <int NT_MAX>        // tiles per wavefront: V <= 16 * 64 * NT_MAX
 __global__ __launch_bounds__(SNT) void nucleus_kernel(const float* __restrict__ logits, const uint64_t* __restrict__ sorted,
                                                       int V, const double* __restrict__ top_p,
                                                       const double* __restrict__ temp, const int32_t* __restrict__ top_k,
@@ -149,57 +167,98 @@ __global__ __launch_bounds__(SNT) void nucleus_kernel(const float* __restrict__ 
                                                       int64_t ld_tokens, int32_t* __restrict__ pos,
                                                       const int32_t* __restrict__ pos_start,
                                                       uint8_t* __restrict__ keep_mask, float* __restrict__ filtered,
-                                                      float* __restrict__ fsorted, const mtj_next_embed ne) {
+                                                      const mtj_next_embed ne) {
   __shared__ double sh[SNT / 64];
   __shared__ int sh_i[SNT / 64];
   __shared__ int chosen;
-  const int b = blockIdx.x, tid = threadIdx.x;
+  const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint64_t* srt = sorted + (int64_t)b * V;
-  float* fs = fsorted + (int64_t)b * V;           // filtered logits in sorted order
-  const int per = (V + SNT - 1) / SNT;
-  const int j0 = tid * per, j1 = (j0 + per < V) ? j0 + per : V;
+  const int nt = (V + SNT - 1) / SNT;             // tiles per wavefront (uniform), <= NT_MAX
+  const int jw = wave * nt * 64 + lane;           // my rank in tile 0
   const int step = pos[b] - pos_start[b];
   const double tp = top_p[b], tmp = temp[b], u = uniforms[(int64_t)b * ld_u + step];
   const int kk = top_k ? top_k[b] : 0x7fffffff;
 
-  // ---- softmax of the sorted logits (max is element 0) and its running sum
+  float val[NT_MAX];                              // sorted logits of my ranks (-inf beyond V)
+  uint32_t idp[NT_MAX / 2];                       // their token ids, two per register
+#pragma unroll
+  for (int t = 0; t < NT_MAX; ++t) {
+    val[t] = -INFINITY;
+    if ((t & 1) == 0) idp[t / 2] = 0;
+    if (t < nt) {
+      const int j = jw + t * 64;
+      if (j < V) {
+        const uint64_t key = srt[j];
+        val[t] = key_value(key);
+        idp[t / 2] |= (uint32_t)(key & 0xffffu) << (16 * (t & 1));
+      }
+    }
+  }
+  auto id_of = [&](int t) { return (idp[t / 2] >> (16 * (t & 1))) & 0xffffu; };
+
+  // ---- softmax of the sorted logits (the maximum is rank 0)
   const double l0 = (double)key_value(srt[0]);
   double loc = 0.0;
-  for (int j = j0; j < j1; ++j) loc += exp((double)key_value(srt[j]) - l0);
-  const double Z = block_sum(loc, sh);
-  double run = block_exclusive(loc / Z, sh);      // mass strictly before j0
+#pragma unroll
+  for (int t = 0; t < NT_MAX; ++t)
+    if (t < nt) loc += (jw + t * 64 < V) ? exp((double)val[t] - l0) : 0.0;
+  const double Z = block_sum(loc, sh);            // leaves the per-wavefront sums in sh
+  double base = 0.0;                              // mass of the ranks before my wavefront's
+  for (int w = 0; w < wave; ++w) base += sh[w] / Z;
+  __syncthreads();
+
   // ---- filter: remove rank j when the mass of ranks [0, j-1] already exceeds top_p (sampling.py:28-30)
+  uint64_t removed = 0;                           // bit t: my rank of tile t is outside the nucleus
   double tmax = -INFINITY;
-  for (int j = j0; j < j1; ++j) {
-    const uint64_t key = srt[j];
-    const uint32_t id = (uint32_t)(key & 0xffffu);
-    const float l = logits[(int64_t)b * V + id];   // the original bits (keeps -0.0)
-    const bool rm = (j > 0) && (run > tp);
-    run += exp((double)key_value(key) - l0) / Z;
+  auto filtered_of = [&](int t, uint32_t id, float l) {
     float f = l;
-    if (j >= kk) f = sub_product(f, 1e10f, (float)id);   // top-k quirk: subtracts 1e10 * token id
-    f = f - (rm ? 1e10f : 0.0f);
-    fs[j] = f;
-    if (filtered) filtered[(int64_t)b * V + id] = f;
-    if (keep_mask) keep_mask[(int64_t)b * V + id] = (f == l) ? 1 : 0;
-    tmax = fmax(tmax, (double)f / tmp);
+    if (jw + t * 64 >= kk) f = sub_product(f, 1e10f, (float)id);   // top-k quirk: subtracts 1e10 * token id
+    return f - (((removed >> t) & 1) ? 1e10f : 0.0f);
+  };
+#pragma unroll
+  for (int t = 0; t < NT_MAX; ++t) {
+    if (t < nt) {
+      const int j = jw + t * 64;
+      const bool live = j < V;
+      const double e = live ? exp((double)val[t] - l0) / Z : 0.0;
+      const double incl = wave_inclusive(e);
+      const double before = base + (incl - e);
+      if (live && j > 0 && before > tp) removed |= 1ull << t;
+      base += __shfl(incl, 63);
+      if (live) {
+        const uint32_t id = id_of(t);
+        // the sort key folds -0.0 into +0.0: fetch the original bits for a zero
+        const float l = (val[t] == 0.0f) ? logits[(int64_t)b * V + id] : val[t];
+        const float f = filtered_of(t, id, l);
+        if (filtered) filtered[(int64_t)b * V + id] = f;
+        if (keep_mask) keep_mask[(int64_t)b * V + id] = (f == l) ? 1 : 0;
+        tmax = fmax(tmax, (double)f / tmp);
+      }
+    }
   }
   tmax = block_max(tmax, sh);
   // ---- inverse-CDF draw over exp(filtered / temp - max) in sorted order
   double wloc = 0.0;
-  for (int j = j0; j < j1; ++j) wloc += exp((double)fs[j] / tmp - tmax);
+#pragma unroll
+  for (int t = 0; t < NT_MAX; ++t)
+    if (t < nt && jw + t * 64 < V) wloc += exp((double)filtered_of(t, id_of(t), val[t]) / tmp - tmax);
   const double total = block_sum(wloc, sh);
-  double cum = block_exclusive(wloc, sh);
+  double cum = 0.0;
+  for (int w = 0; w < wave; ++w) cum += sh[w];
   const double target = u * total;
   int first = 0x7fffffff, lastpos = -1;
-  for (int j = j0; j < j1; ++j) {
-    const double w = exp((double)fs[j] / tmp - tmax);
-    cum += w;
-    if (w > 0.0) lastpos = j;
-    if (cum > target && first == 0x7fffffff) first = j;
+#pragma unroll
+  for (int t = 0; t < NT_MAX; ++t) {
+    if (t < nt) {
+      const int j = jw + t * 64;
+      const double w = (j < V) ? exp((double)filtered_of(t, id_of(t), val[t]) / tmp - tmax) : 0.0;
+      const double incl = wave_inclusive(w);
+      if (w > 0.0) lastpos = j;
+      if (cum + incl > target && j < V && first == 0x7fffffff) first = j;
+      cum += __shfl(incl, 63);
+    }
   }
   // min over first, max over lastpos
-  const int lane = tid & 63, wave = tid >> 6;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     first = min(first, __shfl_xor(first, o));
@@ -223,19 +282,17 @@ __global__ __launch_bounds__(SNT) void nucleus_kernel(const float* __restrict__ 
 }
 
 struct sample_layout {
-  size_t keys_in, keys_out, fsorted, offsets, sort_temp, total;
+  size_t keys_in, keys_out, sort_temp, total;
 };
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-// rocPRIM's scratch need for B segments of V 64-bit keys; fixed upper bound so that the size query does
-// not need a device: the segmented sort asks for a partition scratch of a few words per segment.
+// rocPRIM's merge sort needs one more buffer of keys plus a few words per block; a fixed upper bound, so that
+// the size query does not need a device.
 sample_layout layout(int64_t B, int64_t V) {
   sample_layout L;
   size_t o = 0;
   L.keys_in = o;  o += align256((size_t)B * V * 8);
   L.keys_out = o; o += align256((size_t)B * V * 8);
-  L.fsorted = o;  o += align256((size_t)B * V * 4);
-  L.offsets = o;  o += align256((size_t)(B + 1) * 4);
   L.sort_temp = o; o += align256((size_t)B * V * 8 + (size_t)B * 64 + (1 << 16));
   L.total = o;
   return L;
@@ -272,7 +329,7 @@ extern "C" int mtj_sample_nucleus(const float* logits, int64_t B, int64_t V, con
                                   void* stream) {
   MTJ_REQUIRE(logits && top_p && temp && uniforms && tok && pos && pos_start && work, MTJ_EINVAL,
               "mtj_sample_nucleus: null pointer");
-  MTJ_REQUIRE(B > 0 && V > 0 && V <= 65536 && B * V < (1ll << 31), MTJ_EINVAL,
+  MTJ_REQUIRE(B > 0 && B <= 32768 && V > 0 && V <= 65536 && B * V < (1ll << 31), MTJ_EINVAL,
               "mtj_sample_nucleus: V=%lld must be <= 65536 (token id shares the sort key)", (long long)V);
   MTJ_REQUIRE((reinterpret_cast<uintptr_t>(work) & 255u) == 0, MTJ_EALIGN, "mtj_sample_nucleus: work must be 256-byte aligned");
   mtj_next_embed ne;
@@ -282,21 +339,20 @@ extern "C" int mtj_sample_nucleus(const float* logits, int64_t B, int64_t V, con
   unsigned char* w = reinterpret_cast<unsigned char*>(work);
   uint64_t* kin = reinterpret_cast<uint64_t*>(w + L.keys_in);
   uint64_t* kout = reinterpret_cast<uint64_t*>(w + L.keys_out);
-  float* fsorted = reinterpret_cast<float*>(w + L.fsorted);
-  uint32_t* off = reinterpret_cast<uint32_t*>(w + L.offsets);
   const int64_t total = B * V;
-  make_keys_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(logits, total, (int)V, kin);
-  offsets_kernel<<<(unsigned)((B + 1 + 255) / 256), 256, 0, s>>>(off, (int)B, (int)V);
+  make_keys_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(logits, total, (int)V, (int)B, kin);
   size_t need = 0;
-  hipError_t e = rocprim::segmented_radix_sort_keys_desc(nullptr, need, kin, kout, (unsigned)total, (unsigned)B, off,
-                                                         off + 1, 0, 48, s, false);
+  hipError_t e = rocprim::merge_sort(nullptr, need, kin, kout, (size_t)total, key_desc(), s, false);
   if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_sample_nucleus: sort size query: %s", hipGetErrorString(e));
   const size_t have = L.total - L.sort_temp;
   MTJ_REQUIRE(need <= have, MTJ_ELIMIT, "mtj_sample_nucleus: sort scratch %zu > reserved %zu", need, have);
-  e = rocprim::segmented_radix_sort_keys_desc(w + L.sort_temp, need, kin, kout, (unsigned)total, (unsigned)B, off,
-                                              off + 1, 0, 48, s, false);
+  e = rocprim::merge_sort(w + L.sort_temp, need, kin, kout, (size_t)total, key_desc(), s, false);
   if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_sample_nucleus: sort: %s", hipGetErrorString(e));
-  nucleus_kernel<<<(unsigned)B, SNT, 0, s>>>(logits, kout, (int)V, top_p, temp, top_k, uniforms, ld_u, tok, out_tokens,
-                                             ld_tokens, pos, pos_start, keep_mask, filtered, fsorted, ne);
+  if (V <= SNT * 50)      // GPT-J's 50400-entry vocabulary: everything stays in registers
+    nucleus_kernel<50><<<(unsigned)B, SNT, 0, s>>>(logits, kout, (int)V, top_p, temp, top_k, uniforms, ld_u, tok, out_tokens,
+                                                   ld_tokens, pos, pos_start, keep_mask, filtered, ne);
+  else
+    nucleus_kernel<64><<<(unsigned)B, SNT, 0, s>>>(logits, kout, (int)V, top_p, temp, top_k, uniforms, ld_u, tok, out_tokens,
+                                                   ld_tokens, pos, pos_start, keep_mask, filtered, ne);
   return mtj_check_launch("mtj_sample_nucleus");
 }

@@ -333,6 +333,8 @@ def nucleaus_filter(logits: np.ndarray, top_p=0.9, top_k=None, acc=np.float64) -
     The softmax and its running sum are evaluated in `acc` precision; the contract
     shared with the HIP kernel is acc=float64 (a keep/remove decision then differs from
     the exact real-number result only if a cumulative mass lies within ~1e-15 of top_p).
+    top_p == 1.0 exactly is such a case by construction (the total mass is 1 up to rounding, so
+    tail tokens may be removed depending on summation order); "keep everything" is top_p > 1.
     Returns the filtered float32 logits in token order."""
     logits = np.array(logits, np.float32, copy=True)
     assert logits.ndim == 2

@@ -186,6 +186,14 @@ class Engine:
             self.layer_prefill(ses, i, x, h, act, Tp, ses.pos0)
         return x
 
+    def project(self, ses, x, out):
+        """ProjectionShard.__call__ (layers.py:561-567) on every row of x: out [M, V] float32."""
+        L, w, s = _abi.lib(), self.w, _abi.stream_handle()
+        M, d, V = x.shape[0], w.d, w.V
+        h = ses.h_pf[:M]
+        check(L.mtj_layernorm(ptr(x), ptr(w.pln_s), ptr(w.pln_o), M, d, ptr(h), w.dtype, s))
+        check(L.mtj_gemm(ptr(h), d, ptr(w.w_p), ptr(w.b_p), M, V, d, w.dtype, EPI_STORE, ptr(out), V, F32, None, s))
+
     def layer_prefill(self, ses, i, x, h, act, Tp, pos0):
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()
         M, d, F = x.shape[0], w.d, w.F

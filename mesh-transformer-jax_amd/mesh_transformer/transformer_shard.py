@@ -193,6 +193,42 @@ class CausalTransformer:
                 out = out + (masks.permute(1, 0, 2).cpu().numpy().astype(bool),)
             return final_state, out
 
+    # ------------------------------------------------------------------ full forward
+    def forward(self, ctx, ctx_length=None, timing=None):
+        """Logits at every position: embed -> layers -> ProjectionShard, the composition of
+        transformer_shard.py:47-62 without the loss (the full-context prefill with the 50400-wide projection).
+
+        ctx [B, L] token ids, left-padded when ctx_length [B] is given.  Returns a float32 torch tensor
+        [B, Tp, V] on the GPU with Tp = max(ctx_length) (= L without padding); row t of sequence b belongs to
+        ctx[b, L - Tp + t], rows of padding are zero.  `timing`, a dict, receives forward_s and tokens."""
+        eng = self.engine()
+        ctx = np.ascontiguousarray(np.asarray(ctx)).astype(np.int64)
+        if ctx.ndim != 2:
+            raise ValueError("ctx must be [batch, length]")
+        B, Lc = ctx.shape
+        P = np.full(B, Lc, np.int64) if ctx_length is None else np.asarray(ctx_length).astype(np.int64).reshape(-1)
+        if P.shape[0] != B or P.min() < 1 or P.max() > Lc:
+            raise ValueError("ctx_length needs one entry per sequence, each in [1, ctx length]")
+        Tp = int(P.max())
+        dev = self.device
+        with torch.cuda.device(dev):
+            ses = eng.session(B, Tp, Tp, Tp + 1)
+            ses.pos0.copy_(torch.from_numpy((-(Tp - P)).astype(np.int32)))
+            rect = torch.from_numpy(np.ascontiguousarray(ctx[:, Lc - Tp:]).astype(np.int32)).to(dev)
+            logits = torch.empty(B * Tp, eng.w.V, dtype=torch.float32, device=dev)
+            torch.cuda.synchronize(dev)
+            t0 = time.perf_counter()
+            x = eng.prefill(ses, rect, Tp)
+            eng.project(ses, x, logits)
+            torch.cuda.synchronize(dev)
+            if timing is not None:
+                timing.update(forward_s=time.perf_counter() - t0, tokens=int(P.sum()))
+            logits = logits.view(B, Tp, eng.w.V)
+            if int(P.min()) < Tp:
+                pad = torch.arange(Tp, device=dev)[None, :] < torch.from_numpy(Tp - P).to(dev)[:, None]
+                logits[pad] = 0.0
+            return logits
+
     def _ensure_io(self, ses, G, V):
         if getattr(ses, "G_max", 0) < G:
             dev = self.device

@@ -142,6 +142,36 @@ def test_batched_ragged_nucleus_bit_exact_given_logits():
     assert np.array_equal(out2[0], toks)
 
 
+def test_forward_logits_every_position():
+    """CausalTransformer.forward (embed -> layers -> projection at every position) against the oracle's full
+    forward: fp32 within 1e-4 relative; left padding leaves the real rows unchanged and zeroes the padded ones;
+    bf16 within the 2e-2 logit tolerance."""
+    from mesh_transformer import sampling
+    params = O.seeded_params(CFG1, 0)
+    toks = O.seeded_prompt(5, 2, 70)
+    net = net_for(CFG1, params, sampling.greedy_sample)
+    got = net.forward(toks)
+    assert got.shape == (2, 70, CFG1["n_vocab"]) and got.dtype == torch.float32
+    m = O.Model(CFG1, params, torch.float64)
+    for b in range(2):
+        assert rel(got[b], m.forward(toks[b])) < 1e-4
+    # ragged: sequence 1 keeps only its last 33 tokens, left-padded
+    ctx = toks.copy()
+    ctx[1, :37] = 0
+    got2 = net.forward(ctx, [70, 33])
+    assert rel(got2[0], m.forward(toks[0])) < 1e-4
+    assert rel(got2[1, 37:], m.forward(toks[1, 37:])) < 1e-4
+    assert float(got2[1, :37].abs().max()) == 0.0
+    # bf16 weights, d_head 256
+    pb = O.seeded_params(CFG_BF, 1, torch.bfloat16)
+    tb = O.seeded_prompt(6, 1, 96)
+    gb = net_for(CFG_BF, pb, sampling.greedy_sample).forward(tb)
+    refb = O.Model(CFG_BF, pb, torch.float64).forward(tb[0])
+    assert float((gb[0].double().cpu() - refb).abs().max()) < 2e-2
+    with pytest.raises(ValueError):
+        net.forward(toks, [70, 71])
+
+
 def test_sliding_window_evicts_oldest_tokens():
     """ctx not padded (L == P): every decode step drops the oldest real token (layers.py:325-326)."""
     from mesh_transformer import sampling

@@ -67,7 +67,7 @@ template <typename T, int DH, int NW, int BKV>
 __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ kc,
                                                                const T* __restrict__ vt, const int32_t* __restrict__ pos0,
                                                                int H, int Tp, int Tcap, int64_t ldvt, T* __restrict__ out,
-                                                               int64_t ld_out) {
+                                                               int64_t ld_out, int nseq, int nqblk) {
   constexpr int NT = NW * 64;
   constexpr int BQ = NW * 32;
   constexpr int EPC = mma<T>::EPC;
@@ -86,8 +86,12 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 31, fg = lane >> 5;
-  const int h = blockIdx.y, b = blockIdx.z;
-  const int qt0 = (gridDim.x - 1 - blockIdx.x) * BQ;   // longest (latest) query blocks are dispatched first
+  // Workgroups are dispatched in blockIdx.x order: the head / sequence index varies fastest and the query block
+  // slowest, latest block first, so that the longest workgroups of ALL heads start first and the tail of the
+  // launch consists of short ones.
+  const int hb = blockIdx.x % (H * nseq), qblk = blockIdx.x / (H * nseq);
+  const int h = hb % H, b = hb / H;
+  const int qt0 = (nqblk - 1 - qblk) * BQ;
   const int p0 = pos0[b];                       // <= 0: minus the number of padding rows
   const int t = qt0 + wave * 32 + fr;           // this lane's query (rectangle index)
   const int qpos = (t < Tp) ? t + p0 : -1;      // its position; < 0 = padding / out of range
@@ -482,10 +486,11 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
       if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_attn_prefill: hipFuncSetAttribute: %s", hipGetErrorString(e)); \
       attr_set = true;                                                                                               \
     }                                                                                                                \
-    dim3 grid((unsigned)((Tp + NW * 32 - 1) / (NW * 32)), (unsigned)H, (unsigned)B);                                 \
-    attn_prefill_kernel<T, DH, NW, BKV><<<grid, NW * 64, lds, s>>>((const T*)q, (const T*)k_cache, (const T*)v_t,    \
-                                                                  pos0, (int)H, (int)Tp, (int)Tcap, ldvt, (T*)out,   \
-                                                                  ld_out); \
+    const int64_t nqblk = (Tp + NW * 32 - 1) / (NW * 32);                                                            \
+    MTJ_REQUIRE(nqblk * H * B < (1ll << 31), MTJ_ELIMIT, "mtj_attn_prefill: too many workgroups");                    \
+    attn_prefill_kernel<T, DH, NW, BKV><<<(unsigned)(nqblk * H * B), NW * 64, lds, s>>>(                              \
+        (const T*)q, (const T*)k_cache, (const T*)v_t, pos0, (int)H, (int)Tp, (int)Tcap, ldvt, (T*)out, ld_out,      \
+        (int)B, (int)nqblk);                                                                                         \
   } while (0)
   if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL(bf16_t, 256, 4, 32);
   else if (dtype == MTJ_BF16 && dh == 64) MTJ_PREFILL(bf16_t, 64, 8, 64);

@@ -172,6 +172,42 @@ def test_forward_logits_every_position():
         net.forward(toks, [70, 71])
 
 
+def test_config1_against_the_committed_fixture():
+    """BASELINE config 1 against tests/golden/config1_greedy.npz: tokens identical, top-8 logits of every step
+    within 1e-4 relative, logit checksums."""
+    import os
+    from mesh_transformer import sampling
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "config1_greedy.npz"))
+    net = net_for(CFG1, O.seeded_params(CFG1, 0), sampling.greedy_sample)
+    ctx = O.left_pad(g["prompt"], 168)
+    _, out = net.generate(ctx, [128], 32, {}, return_logits=True)
+    assert np.array_equal(out[0][0, :, 0], g["tokens"])
+    lg = out[2][0, :, 0, :].astype(np.float64)
+    got_top = np.take_along_axis(lg, g["top8_ids"].astype(np.int64), -1)
+    assert np.abs(got_top - g["top8_logits"]).max() <= 1e-4 * np.abs(g["top8_logits"]).max()
+    np.testing.assert_allclose(lg.sum(-1), g["logits_sum"], rtol=0, atol=1e-4 * np.sqrt(g["logits_sqsum"]).max())
+    np.testing.assert_allclose((lg ** 2).sum(-1), g["logits_sqsum"], rtol=2e-4)
+
+
+def test_generate_from_an_8_shard_checkpoint(tmp_path):
+    """resharding_example.py:40-60: network.state = read_ckpt(network.state, dir, 8, shards_out=1), then generate."""
+    import os
+    from oracle import ckpt_oracle as CK
+    from mesh_transformer import checkpoint, sampling
+    params = O.seeded_params(CFG1, 7)
+    d = str(tmp_path) + os.sep
+    stacked = {"params": CK.shard_tree(params, 8, CFG1), "step": np.full(8, 5, np.uint32)}
+    for s in range(8):
+        checkpoint.write_ckpt(stacked, d, s)
+    net = net_for(CFG1, None, sampling.greedy_sample)            # random init, then the checkpoint replaces it
+    net.state = checkpoint.read_ckpt(net.state, d, 8, shards_out=1)
+    prompt = O.seeded_prompt(8, 1, 24)
+    ctx = O.left_pad(prompt, 48)
+    _, out = net.generate(ctx, [24], 8, {})
+    ref = O.Model(CFG1, params, torch.float64).generate(ctx, [24], 8, O.greedy_sample, {})
+    assert np.array_equal(out[0], ref[0])
+
+
 def test_sliding_window_evicts_oldest_tokens():
     """ctx not padded (L == P): every decode step drops the oldest real token (layers.py:325-326)."""
     from mesh_transformer import sampling

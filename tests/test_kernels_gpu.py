@@ -443,6 +443,21 @@ def test_nucleus_bit_exact_vs_oracle(L, V, spread):
             assert tok[r] == O.inverse_cdf_draw(logits[r:r + 1], f_ref, float(temp[r]), float(u[r])), (V, spread, r, k)
 
 
+def test_nucleus_against_the_committed_fixture(L):
+    """tests/golden/nucleus_cases.npz: keep-masks and tokens bit for bit."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "nucleus_cases.npz"))
+    V = g["logits"].shape[1]
+    keep = np.unpackbits(g["keep"], axis=-1)[:, :V].astype(bool)
+    for r in range(g["logits"].shape[0]):
+        k = None if g["top_k"][r] == 0 else np.array([g["top_k"][r]], np.int32)
+        tok, mask, _ = _sample(L, g["logits"][r:r + 1], g["top_p"][r], g["temp"][r], k, g["u"][r])
+        assert np.array_equal(mask[0], keep[r]), r
+        assert tok[0] == g["token"][r], r
+    _, mask, _ = _sample(L, g["demo"], 0.9, 1.0, None, 0.5)
+    assert np.array_equal(mask[0], g["demo_keep"])
+
+
 def test_greedy_lowest_index_on_ties(L):
     a = abi()
     V = 50400

@@ -4,6 +4,9 @@ independent GPT-J implementation in `transformers` built from a local config obj
 import itertools
 import math
 
+import os
+import sys
+
 import numpy as np
 import pytest
 import torch
@@ -293,3 +296,24 @@ def test_inverse_cdf_draw_brute_force_and_chi_square():
 
 def test_greedy_lowest_index_on_ties():
     assert O.greedy_sample(None, np.array([[1.0, 3.0, 3.0, 2.0]], np.float32)) == 1
+
+
+# ---------------------------------------------------------------------------- committed fixtures
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def test_golden_fixtures_match_the_oracle():
+    """tests/golden/*.npz (written by tests/golden/make_golden.py) are what the oracle computes today."""
+    sys.path.insert(0, GOLDEN)
+    import make_golden as G
+    for name, fn in (("config1_greedy.npz", G.config1), ("nucleus_cases.npz", G.nucleus)):
+        want = np.load(os.path.join(GOLDEN, name))
+        got = fn()
+        assert sorted(want.files) == sorted(got)
+        for k in want.files:
+            if want[k].dtype.kind == "f":
+                np.testing.assert_allclose(got[k], want[k], rtol=1e-9, atol=1e-12, err_msg=f"{name}:{k}")
+            else:
+                assert np.array_equal(got[k], want[k]), f"{name}:{k}"
+    demo = np.load(os.path.join(GOLDEN, "nucleus_cases.npz"))
+    assert set(np.nonzero(~demo["demo_keep"])[0].tolist()) == {0, 1, 11}      # hand-worked, sampling.py:49

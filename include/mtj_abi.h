@@ -94,6 +94,13 @@ int mtj_embed(const int32_t* tok, int64_t M, const void* W, const float* b, int6
 int mtj_layernorm(const float* x, const float* scale, const float* offset, int64_t M, int64_t d,
                   void* out, int out_dtype, void* stream);
 
+/* Per-row cross entropy of float32 logits [M, V] (row stride ld) against int32 targets [M]:
+ * ProjectionShard.loss, layers.py:569-593, on one shard: loss = log(sum exp(l - max)) - (l[target] - max),
+ * correct = (l[target] == max).  A target outside [0, V) selects nothing (loss = log-sum-exp), like an all-zero
+ * one-hot row.  correct may be NULL. */
+int mtj_xent(const float* logits, int64_t ld, const int32_t* target, int64_t M, int64_t V, float* loss,
+             uint8_t* correct, void* stream);
+
 /* C = A[M, K] (dtype, row stride lda) x W[N, K]^T (packed, dtype) with epilogue `epi`.
  * hk.Linear call sites: layers.py:249-258, 559.  MFMA kernel; bias is float32 [N] or NULL.
  * STORE: out [M, ldo] in out_dtype.  RESID: out float32 [M, ldo].  INPROJ: `ip` non-NULL, bias = b1 [F]. */
@@ -123,10 +130,12 @@ int mtj_gemv(const float* x, const float* ln_scale, const float* ln_offset, cons
  * layers.py:260-285, 347-366).  q [B,H,Tp,dh], k_cache [B,H,Tcap,dh] (rotated), v_t [B,H,dh,ldvt] with
  * ldvt >= Tp rounded up to a multiple of 64 (columns beyond the last key may hold anything);
  * out[m, h*dh + c] with row stride ld_out, dtype.  Scores are divided by sqrt(dh) after the dot;
- * masked keys contribute exactly 0 (exp(-1e10 - max) underflows in float32).  Padding rows get zeros. */
+ * masked keys contribute exactly 0 (exp(-1e10 - max) underflows in float32).  Padding rows get zeros.
+ * key_limit (may be NULL): int32 [B]; query position p of sequence b sees keys 0 .. min(p, key_limit[b]) - the
+ * additive mask (arange > ctx_length) * -1e10 of the evaluation path, transformer_shard.py:130. */
 int mtj_attn_prefill(const void* q, const void* k_cache, const void* v_t, const int32_t* pos0, int64_t B,
                      int64_t H, int64_t Tp, int64_t Tcap, int64_t dh, int64_t ldvt, void* out, int64_t ld_out,
-                     int dtype, void* stream);
+                     int dtype, const int32_t* key_limit, void* stream);
 
 /* One-token attention over the K/V window (decode_once, layers.py:316-344): for sequence b the valid
  * slots are [0, min(pos[b]+1, Tcap)).  q float32 [B,H,dh]; caches in `dtype`; out [B, ld_out] in out_dtype

@@ -67,7 +67,8 @@ template <typename T, int DH, int NW, int BKV>
 __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ kc,
                                                                const T* __restrict__ vt, const int32_t* __restrict__ pos0,
                                                                int H, int Tp, int Tcap, int64_t ldvt, T* __restrict__ out,
-                                                               int64_t ld_out, int nseq, int nqblk) {
+                                                               int64_t ld_out, int nseq, int nqblk,
+                                                               const int32_t* __restrict__ key_limit) {
   constexpr int NT = NW * 64;
   constexpr int BQ = NW * 32;
   constexpr int EPC = mma<T>::EPC;
@@ -95,12 +96,16 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
   const int p0 = pos0[b];                       // <= 0: minus the number of padding rows
   const int t = qt0 + wave * 32 + fr;           // this lane's query (rectangle index)
   const int qpos = (t < Tp) ? t + p0 : -1;      // its position; < 0 = padding / out of range
+  // last key this query may see: itself, or an earlier position when the caller masks the tail of the sequence
+  const int klim = key_limit ? key_limit[b] : 0x7fffffff;
+  const int qsee = qpos < klim ? qpos : klim;
   const int last_t = (qt0 + BQ - 1 < Tp - 1) ? qt0 + BQ - 1 : Tp - 1;
   const int kmax = last_t + p0;                 // last key any query of this workgroup may see
   const int klast = Tp - 1 + p0;                // last key position that exists for this sequence
   const int wave_last = qt0 + wave * 32 + 31 + p0;   // last key this wavefront may see
   // first query position of this wavefront if all 32 of its queries are real, else -1 (always mask)
-  const int wave_first = (qt0 + wave * 32 + 31 < Tp) ? qt0 + wave * 32 + p0 : -1;
+  const int wave_first0 = (qt0 + wave * 32 + 31 < Tp) ? qt0 + wave * 32 + p0 : -1;
+  const int wave_first = wave_first0 < klim ? wave_first0 : klim;
   const int64_t bh = (int64_t)b * H + h;
 
   // Q fragments (B operand of S^T): lane (query fr, half fg) holds Q[t][ks*16 + fg*8 .. +8)
@@ -226,7 +231,7 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             const int key = key0 + kb * 32 + 16 * (v / 8) + 8 * fg + (v % 8);
-            s[kb][v] = (key <= qpos) ? s[kb][v] * sc2 : -INFINITY;
+            s[kb][v] = (key <= qsee) ? s[kb][v] * sc2 : -INFINITY;
             mt = fmaxf(mt, s[kb][v]);
           }
       }
@@ -464,7 +469,7 @@ int decode_splits(int64_t Tcap) { return (int)((Tcap + DEC_CHUNK - 1) / DEC_CHUN
 
 extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* v_t, const int32_t* pos0, int64_t B,
                                 int64_t H, int64_t Tp, int64_t Tcap, int64_t dh, int64_t ldvt, void* out,
-                                int64_t ld_out, int dtype, void* stream) {
+                                int64_t ld_out, int dtype, const int32_t* key_limit, void* stream) {
   MTJ_REQUIRE(q && k_cache && v_t && pos0 && out, MTJ_EINVAL, "mtj_attn_prefill: null pointer");
   MTJ_REQUIRE(B > 0 && H > 0 && Tp > 0 && Tp <= Tcap && ld_out >= H * dh && B < 65536 && H < 65536, MTJ_EINVAL,
               "mtj_attn_prefill: bad shape B=%lld H=%lld Tp=%lld Tcap=%lld", (long long)B, (long long)H,
@@ -490,7 +495,7 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
     MTJ_REQUIRE(nqblk * H * B < (1ll << 31), MTJ_ELIMIT, "mtj_attn_prefill: too many workgroups");                    \
     attn_prefill_kernel<T, DH, NW, BKV><<<(unsigned)(nqblk * H * B), NW * 64, lds, s>>>(                              \
         (const T*)q, (const T*)k_cache, (const T*)v_t, pos0, (int)H, (int)Tp, (int)Tcap, ldvt, (T*)out, ld_out,      \
-        (int)B, (int)nqblk);                                                                                         \
+        (int)B, (int)nqblk, key_limit);                                                                                       \
   } while (0)
   if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL(bf16_t, 256, 4, 32);
   else if (dtype == MTJ_BF16 && dh == 64) MTJ_PREFILL(bf16_t, 64, 8, 64);

@@ -158,3 +158,42 @@ extern "C" int mtj_layernorm(const float* x, const float* scale, const float* of
     return mtj_fail(MTJ_EDTYPE, "mtj_layernorm: out_dtype %d", out_dtype);
   return mtj_check_launch("mtj_layernorm");
 }
+
+// ---------------------------------------------------------------- cross entropy of a logits row
+// ProjectionShard.loss (layers.py:569-593) on one shard: logits -= max; loss = log(sum exp) - logits[target];
+// correct = (logits[target] == 0), i.e. the target holds the row maximum.  One 256-thread workgroup per row.
+__global__ __launch_bounds__(256) void xent_kernel(const float* __restrict__ logits, const int32_t* __restrict__ target,
+                                                   int64_t ld, int V, float* __restrict__ loss,
+                                                   uint8_t* __restrict__ correct) {
+  __shared__ float red[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const float* row = logits + (int64_t)blockIdx.x * ld;
+  float m = -INFINITY;
+  for (int i = tid; i < V; i += 256) m = fmaxf(m, row[i]);
+  m = wave_max(m);
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  float s = 0.f;
+  for (int i = tid; i < V; i += 256) s += expf(row[i] - m);
+  s = wave_sum(s);
+  if (lane == 0) red[wave] = s;
+  __syncthreads();
+  if (tid == 0) {
+    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    const int t = target[blockIdx.x];
+    const float pred = ((uint32_t)t < (uint32_t)V) ? row[t] - m : 0.f;    // an all-zero one-hot row selects nothing
+    loss[blockIdx.x] = logf(total) - pred;
+    if (correct) correct[blockIdx.x] = (pred == 0.f) ? 1 : 0;
+  }
+}
+
+extern "C" int mtj_xent(const float* logits, int64_t ld, const int32_t* target, int64_t M, int64_t V, float* loss,
+                        uint8_t* correct, void* stream) {
+  MTJ_REQUIRE(logits && target && loss, MTJ_EINVAL, "mtj_xent: null pointer");
+  MTJ_REQUIRE(M > 0 && M < (1ll << 31) && V > 0 && V < (1ll << 31) && ld >= V, MTJ_EINVAL,
+              "mtj_xent: bad shape M=%lld V=%lld ld=%lld", (long long)M, (long long)V, (long long)ld);
+  xent_kernel<<<(unsigned)M, 256, 0, (hipStream_t)stream>>>(logits, target, ld, (int)V, loss, correct);
+  return mtj_check_launch("mtj_xent");
+}

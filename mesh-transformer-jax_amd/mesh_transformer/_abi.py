@@ -40,11 +40,12 @@ SIGNATURES = {
     "mtj_pack_weight": (_i32, [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _i32, _p]),
     "mtj_embed": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i32, _p, _p]),
     "mtj_layernorm": (_i32, [_p, _p, _p, _i64, _i64, _p, _i32, _p]),
+    "mtj_xent": (_i32, [_p, _i64, _p, _i64, _i64, _p, _p, _p]),
     "mtj_gemm": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, C.POINTER(InProj), _p]),
     "mtj_gemm_splitk_work_bytes": (_i64, [_i64, _i64, _i64, _i32]),
     "mtj_gemm_splitk": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, _p, _i64, _p]),
     "mtj_gemv": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p, _i32, C.POINTER(InProj), _p]),
-    "mtj_attn_prefill": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64, _i32, _p]),
+    "mtj_attn_prefill": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64, _i32, _p, _p]),
     "mtj_attn_decode_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "mtj_attn_decode": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _i32, _i32, _p, _p]),
     "mtj_sample_greedy": (_i32, [_p, _i64, _i64, _p, _p, _i64, _p, _p, C.POINTER(NextEmbed), _p]),

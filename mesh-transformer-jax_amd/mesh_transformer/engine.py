@@ -174,7 +174,7 @@ class Engine:
         ip.act, ip.ld_act, ip.act_dtype = ptr(act), act.shape[1], act_dtype
         return ip
 
-    def prefill(self, ses, tokens_rect, Tp):
+    def prefill(self, ses, tokens_rect, Tp, key_limit=None):
         """generate_initial (transformer_shard.py:74-95) on a [B, Tp] right-aligned rectangle; the
         dead logits projection of :95 is not computed."""
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()
@@ -183,7 +183,7 @@ class Engine:
         x, h, act = ses.x_pf[:M], ses.h_pf[:M], ses.act_pf[:M]
         check(L.mtj_embed(ptr(tokens_rect), M, ptr(w.we), ptr(w.be), w.V, d, w.dtype, ptr(x), s))
         for i in w.layer_ids:
-            self.layer_prefill(ses, i, x, h, act, Tp, ses.pos0)
+            self.layer_prefill(ses, i, x, h, act, Tp, ses.pos0, key_limit)
         return x
 
     def project(self, ses, x, out):
@@ -194,7 +194,7 @@ class Engine:
         check(L.mtj_layernorm(ptr(x), ptr(w.pln_s), ptr(w.pln_o), M, d, ptr(h), w.dtype, s))
         check(L.mtj_gemm(ptr(h), d, ptr(w.w_p), ptr(w.b_p), M, V, d, w.dtype, EPI_STORE, ptr(out), V, F32, None, s))
 
-    def layer_prefill(self, ses, i, x, h, act, Tp, pos0):
+    def layer_prefill(self, ses, i, x, h, act, Tp, pos0, key_limit=None):
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()
         M, d, F = x.shape[0], w.d, w.F
         check(L.mtj_layernorm(ptr(x), ptr(w.ln_s[i]), ptr(w.ln_o[i]), M, d, ptr(h), w.dtype, s))
@@ -202,7 +202,7 @@ class Engine:
         check(L.mtj_gemm(ptr(h), d, ptr(w.w_in[i]), ptr(w.b1[i]), M, 3 * d + F, d, w.dtype, EPI_INPROJ,
                          None, 0, 0, C.byref(ip), s))
         check(L.mtj_attn_prefill(ptr(ses.q_pf), ptr(ses.kc[i]), ptr(ses.vt), ptr(pos0), ses.B, self.H, Tp, ses.Tcap,
-                                 self.dh, ses.ldvt, ptr(act), d + F, w.dtype, s))
+                                 self.dh, ses.ldvt, ptr(act), d + F, w.dtype, ptr(key_limit), s))
         check(L.mtj_gemm(ptr(act), d + F, ptr(w.w_out[i]), ptr(w.b2[i]), M, d, d + F, w.dtype, EPI_RESID,
                          ptr(x), d, F32, None, s))
 

@@ -229,6 +229,45 @@ class CausalTransformer:
                 logits[pad] = 0.0
             return logits
 
+    # ------------------------------------------------------------------ evaluation
+    def eval(self, sample):
+        """transformer_shard.py:308-324 with CausalTransformerShard.loss/eval (:47-72, 123-132) and
+        ProjectionShard.loss (layers.py:569-593): per-token cross entropy of sample["target"] [B, T] under the model
+        run on sample["obs"] [B, T]; keys beyond sample["ctx_length"] [B] (default T) are masked for every query.
+        Returns numpy arrays {"loss" [B] (mean over all T positions, as the reference), "last_loss" [B],
+        "all_loss" [B, T], "correct" [B, T] (the target holds the maximum logit)}."""
+        eng = self.engine()
+        obs = np.ascontiguousarray(np.asarray(sample["obs"])).astype(np.int64)
+        tgt = np.ascontiguousarray(np.asarray(sample["target"])).astype(np.int64)
+        if obs.ndim != 2 or tgt.shape != obs.shape:
+            raise ValueError("obs and target must both be [batch, length]")
+        B, T = obs.shape
+        cl = np.asarray(sample["ctx_length"]).astype(np.int64).reshape(-1) if "ctx_length" in sample else np.full(B, T)
+        if cl.shape[0] != B:
+            raise ValueError("ctx_length must have one entry per sequence")
+        dev, L, V = self.device, _abi.lib(), eng.w.V
+        with torch.cuda.device(dev):
+            ses = eng.session(B, T, T, T + 1)
+            ses.pos0.zero_()
+            rect = torch.from_numpy(obs.astype(np.int32)).to(dev)
+            limit = torch.from_numpy(np.minimum(cl, 2 ** 31 - 1).astype(np.int32)).to(dev)
+            target = torch.from_numpy(tgt.astype(np.int32)).to(dev).reshape(-1)
+            x = eng.prefill(ses, rect, T, key_limit=limit)
+            loss = torch.empty(B * T, dtype=torch.float32, device=dev)
+            correct = torch.empty(B * T, dtype=torch.uint8, device=dev)
+            # the logits of a slab of rows at a time: [B*T, V] float32 need not exist all at once
+            rows = max(1, min(B * T, (1 << 30) // (4 * V)))
+            logits = torch.empty(rows, V, dtype=torch.float32, device=dev)
+            for r0 in range(0, B * T, rows):
+                n = min(rows, B * T - r0)
+                eng.project(ses, x[r0:r0 + n], logits[:n])
+                _abi.check(L.mtj_xent(_abi.ptr(logits), V, _abi.ptr(target[r0:r0 + n]), n, V, _abi.ptr(loss[r0:r0 + n]),
+                                      _abi.ptr(correct[r0:r0 + n]), _abi.stream_handle()))
+            torch.cuda.synchronize(dev)
+            all_loss = loss.view(B, T).cpu().numpy()
+            return {"loss": all_loss.mean(-1), "last_loss": all_loss[:, -1].copy(), "all_loss": all_loss,
+                    "correct": correct.view(B, T).cpu().numpy().astype(bool)}
+
     def _ensure_io(self, ses, G, V):
         if getattr(ses, "G_max", 0) < G:
             dev = self.device

@@ -24,6 +24,8 @@ Pinning status (what, other than this file's own formulas, fixes each result):
                              through the reference's own weight-name map
   * decode_once / window   - teacher forcing against the full forward,
                              brute-force sliding window
+  * loss (evaluation)      - torch.nn.functional.cross_entropy and argmax on the
+                             full-forward logits; masked keys cannot influence a row
   * nucleaus_filter        - reference demo vector (sampling.py:49) worked by
                              hand, brute force over prefixes, invariants
   * inverse_cdf_draw       - own contract (the reference's Gumbel draw is
@@ -268,6 +270,22 @@ class Model:
             if taps is not None:
                 taps.append(x.clone())
         return self.proj(x)
+
+    def loss(self, ctx, tgt, ctx_length=None):
+        """CausalTransformerShard.eval/loss (transformer_shard.py:47-72) under the evaluation mask
+        (arange > ctx_length) * -1e10 on the keys (:130), then ProjectionShard.loss (layers.py:569-593) with
+        z_loss = 0: loss = log(sum exp(l - max)) - (l[target] - max), correct = (l[target] - max == 0)."""
+        T = len(ctx)
+        L = T if ctx_length is None else int(ctx_length)
+        mask = (torch.arange(T) > L).to(self.dtype) * -1e10
+        x = self.embed(ctx)
+        for l in self.layers:
+            x = x + l(x, mask)
+        logits = self.proj(x)
+        logits = logits - logits.max(-1, keepdim=True).values
+        pred = logits[torch.arange(T), torch.as_tensor(np.asarray(tgt).astype(np.int64))]
+        all_loss = torch.log(torch.exp(logits).sum(-1)) - pred
+        return {"loss": all_loss.mean(), "last_loss": all_loss[-1], "all_loss": all_loss, "correct": pred == 0.0}
 
     def generate_initial(self, context, length: int, taps: Optional[list] = None):
         """transformer_shard.py:74-95 - prefill on context[:-1]; context[-1] seeds decode."""

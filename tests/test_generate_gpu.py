@@ -189,6 +189,29 @@ def test_config1_against_the_committed_fixture():
     np.testing.assert_allclose((lg ** 2).sum(-1), g["logits_sqsum"], rtol=2e-4)
 
 
+def test_eval_losses_match_the_oracle():
+    """CausalTransformer.eval: per-token cross entropy, `correct`, and the evaluation mask of ragged batches."""
+    from mesh_transformer import sampling
+    params = O.seeded_params(CFG1, 9)
+    net = net_for(CFG1, params, sampling.greedy_sample)
+    rng = np.random.default_rng(1)
+    obs = rng.integers(0, 50257, (3, 40)).astype(np.uint32)
+    tgt = np.roll(obs, -1, axis=1)
+    lens = np.array([40, 17, 1])
+    out = net.eval({"obs": obs, "target": tgt, "ctx_length": lens})
+    m = O.Model(CFG1, params, torch.float64)
+    for b in range(3):
+        ref = m.loss(obs[b], tgt[b], lens[b])
+        assert rel(out["all_loss"][b], ref["all_loss"]) < 1e-4, b
+        assert abs(out["loss"][b] - float(ref["loss"])) < 1e-4 * float(ref["loss"])
+        assert abs(out["last_loss"][b] - float(ref["last_loss"])) < 1e-3
+        assert np.array_equal(out["correct"][b], ref["correct"].numpy())
+    full = net.eval({"obs": obs[:1], "target": tgt[:1]})
+    assert rel(full["all_loss"][0], m.loss(obs[0], tgt[0])["all_loss"]) < 1e-4
+    with pytest.raises(ValueError):
+        net.eval({"obs": obs, "target": tgt[:, :5]})
+
+
 def test_generate_from_an_8_shard_checkpoint(tmp_path):
     """resharding_example.py:40-60: network.state = read_ckpt(network.state, dir, 8, shards_out=1), then generate."""
     import os

@@ -354,7 +354,7 @@ def test_attn_prefill(L, dt, dh, H, Tp):
     ld_out = H * dh + 16
     out = torch.full((B * Tp, ld_out), 7.0, dtype=TD[dt], device=DEV)
     a.check(L.mtj_attn_prefill(a.ptr(q), a.ptr(kc), a.ptr(vt), a.ptr(pos0), B, H, Tp, Tcap, dh, ldvt, a.ptr(out), ld_out,
-                               a.dtype_code(TD[dt]), S()))
+                               a.dtype_code(TD[dt]), None, S()))
     torch.cuda.synchronize()
     for b in range(B):
         pd = pads[b]
@@ -364,6 +364,26 @@ def test_attn_prefill(L, dt, dh, H, Tp):
         assert rel_err(got, ref) < (3e-6 if dt == "f32" else 8e-3), (dt, dh, Tp, b)
         assert float(out[b * Tp:b * Tp + pd, :H * dh].float().abs().max() if pd else 0.0) == 0.0   # padding rows: zeros
     assert torch.all(out[:, H * dh:] == 7.0)
+    # evaluation mask (transformer_shard.py:130): keys beyond key_limit[b] are hidden from every query
+    if Tp >= 33:
+        lim = [Tp // 2, Tp - 1]
+        kl = torch.tensor(lim, dtype=torch.int32, device=DEV)
+        zero = torch.zeros(B, dtype=torch.int32, device=DEV)
+        kc2 = kk.clone()
+        vt2 = torch.zeros(B, H, dh, ldvt, dtype=TD[dt], device=DEV)
+        vt2[:, :, :, :Tp] = vv.permute(0, 1, 3, 2)
+        kcf = torch.zeros(B, H, Tcap, dh, dtype=TD[dt], device=DEV)
+        kcf[:, :, :Tp] = kc2
+        a.check(L.mtj_attn_prefill(a.ptr(q), a.ptr(kcf), a.ptr(vt2), a.ptr(zero), B, H, Tp, Tcap, dh, ldvt, a.ptr(out),
+                                   ld_out, a.dtype_code(TD[dt]), a.ptr(kl), S()))
+        torch.cuda.synchronize()
+        for b in range(B):
+            qq, kq, vq = (t[b].permute(1, 0, 2).double().cpu() for t in (q, kk, vv))
+            sc = torch.einsum("thd,Thd->htT", qq, kq) / math.sqrt(dh)
+            bias = O.MASK * (1.0 - torch.tril(torch.ones(Tp, Tp, dtype=torch.float64)))
+            bias = bias + (torch.arange(Tp) > lim[b]).double() * -1e10
+            ref = torch.einsum("htT,Thd->thd", torch.softmax(sc + bias, -1), vq).reshape(Tp, H * dh)
+            assert rel_err(out[b * Tp:(b + 1) * Tp, :H * dh], ref) < (3e-6 if dt == "f32" else 8e-3), (dt, dh, Tp, b)
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
@@ -456,6 +476,29 @@ def test_nucleus_against_the_committed_fixture(L):
         assert tok[0] == g["token"][r], r
     _, mask, _ = _sample(L, g["demo"], 0.9, 1.0, None, 0.5)
     assert np.array_equal(mask[0], g["demo_keep"])
+
+
+@pytest.mark.parametrize("M,V,ld", [(1, 12, 12), (37, 50400, 50400), (5, 1000, 1024)])
+def test_xent_rows(L, M, V, ld):
+    a = abi()
+    g = torch.Generator().manual_seed(M + V)
+    lg = (torch.randn(M, ld, generator=g) * 3).to(DEV)
+    tgt = torch.randint(0, V, (M,), generator=g).to(torch.int32)
+    tgt[0] = int(lg[0, :V].argmax())                       # a correct one
+    if M > 2:
+        tgt[2] = V + 5                                     # outside the vocabulary: selects nothing
+    tgt = tgt.to(DEV)
+    loss = torch.empty(M, device=DEV)
+    correct = torch.empty(M, dtype=torch.uint8, device=DEV)
+    a.check(L.mtj_xent(a.ptr(lg), ld, a.ptr(tgt), M, V, a.ptr(loss), a.ptr(correct), S()))
+    torch.cuda.synchronize()
+    l64 = lg[:, :V].double()
+    lse = torch.logsumexp(l64, -1)
+    inside = tgt.long() < V
+    ref = lse - torch.where(inside, l64.gather(1, tgt.long().clamp(max=V - 1)[:, None])[:, 0], l64.max(-1).values)
+    assert rel_err(loss, ref) < 2e-6
+    want = (l64.argmax(-1) == tgt.long()) | ~inside         # pred = 0 also when nothing is selected
+    assert torch.equal(correct.bool(), want)
 
 
 def test_greedy_lowest_index_on_ties(L):

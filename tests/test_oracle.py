@@ -298,6 +298,30 @@ def test_greedy_lowest_index_on_ties():
     assert O.greedy_sample(None, np.array([[1.0, 3.0, 3.0, 2.0]], np.float32)) == 1
 
 
+def test_loss_is_cross_entropy_and_the_evaluation_mask_hides_keys():
+    cfg = dict(layers=2, d_model=64, n_heads=4, n_vocab=96, norm="layernorm", pe="rotary", pe_rotary_dims=8,
+               cores_per_replica=1)
+    params = O.seeded_params(cfg, 11)
+    m = O.Model(cfg, params, torch.float64)
+    rng = np.random.default_rng(0)
+    ctx, tgt = rng.integers(0, 96, 24), rng.integers(0, 96, 24)
+    out = m.loss(ctx, tgt)
+    logits = m.forward(ctx)
+    ce = F.cross_entropy(logits, torch.as_tensor(tgt), reduction="none")
+    assert torch.allclose(out["all_loss"], ce, atol=1e-12)
+    assert torch.equal(out["correct"], logits.argmax(-1) == torch.as_tensor(tgt))
+    assert abs(float(out["loss"]) - float(ce.mean())) < 1e-12 and float(out["last_loss"]) == float(out["all_loss"][-1])
+    # ctx_length = 15: rows 0..15 are what they were; keys 16.. are hidden, so tokens 16..22 cannot reach row 23
+    cut = m.loss(ctx, tgt, 15)
+    assert torch.allclose(cut["all_loss"][:16], out["all_loss"][:16], atol=1e-12)
+    assert not torch.allclose(cut["all_loss"][16:], out["all_loss"][16:], atol=1e-6)
+    ctx2 = ctx.copy()
+    ctx2[16:23] = rng.integers(0, 96, 7)
+    cut2 = m.loss(ctx2, tgt, 15)
+    assert abs(float(cut2["all_loss"][23]) - float(cut["all_loss"][23])) < 1e-12
+    assert abs(float(m.loss(ctx2, tgt)["all_loss"][23]) - float(out["all_loss"][23])) > 1e-9
+
+
 # ---------------------------------------------------------------------------- committed fixtures
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 

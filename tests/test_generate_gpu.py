@@ -212,6 +212,23 @@ def test_eval_losses_match_the_oracle():
         net.eval({"obs": obs, "target": tgt[:, :5]})
 
 
+def test_batching_loop_on_the_gpu():
+    """device_serve.py:138-194 around the real network: two requests in a batch of four; with top_p -> 0 the nucleus
+    is the top token alone, so the completions equal the oracle's greedy streams."""
+    from mesh_transformer import sampling, serving
+    cfg = dict(CFG1, n_vocab=2048, seq=40)
+    params = O.seeded_params(cfg, 12)
+    net = net_for(cfg, params, sampling.nucleaus_sample)
+    loop = serving.BatchingLoop(net, seq=40, total_batch=4, gen_length=6)
+    prompts = [O.seeded_prompt(20, 1, 9, hi=2048)[0], O.seeded_prompt(21, 1, 23, hi=2048)[0]]
+    qs = [loop.submit(p.tolist(), 1e-9, 1.0) for p in prompts]
+    assert loop.step() == 2
+    m = O.Model(cfg, params, torch.float64)
+    for p, q in zip(prompts, qs):
+        ref = m.generate(O.left_pad(p[None], 40), [len(p)], 6, O.greedy_sample, {})
+        assert np.array_equal(q.get_nowait(), ref[0][0, :, 0])
+
+
 def test_generate_from_an_8_shard_checkpoint(tmp_path):
     """resharding_example.py:40-60: network.state = read_ckpt(network.state, dir, 8, shards_out=1), then generate."""
     import os

@@ -208,6 +208,9 @@ def main():
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter probe for rocprofv3 --pmc: one plain 234,881,024-byte device copy, then 8 launches "
                          "of the dominant kernel on a 2-layer model of the 6B shape; prints no JSON")
+    ap.add_argument("--prefill-probe", action="store_true",
+                    help="profiling probe: 6 forwards of one full-shape layer on 8 x 2048 tokens (BASELINE config 2) "
+                         "on a 1-layer model of the 6B shape; prints the time per forward, no bench line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the whole model on ONE GPU (no collectives, no sharding); "
@@ -224,6 +227,13 @@ def main():
     dev = torch.device("cuda:0")
     if args.pmc_probe:
         pmc_probe(dev)
+        return
+    if args.prefill_probe:
+        c1 = dict(CFG_6B, layers=1, sampler=sampling.greedy_sample)
+        n1 = CausalTransformer(c1, synthetic_tree(c1, 1, dev, torch.bfloat16))
+        t = time_prefill_layer(n1)
+        fl = 8 * 2048 * (2 * 201326592 + 4 * 4096 * 2049 / 2)
+        print(json.dumps({"layer_8x2048_ms": t * 1e3, "tflops": fl / t / 1e12, "frac_mfma": fl / t / 2.5e15}))
         return
     cfg = dict(CFG_6B, sampler=sampling.greedy_sample)
     K, W = args.steps, args.warmup

@@ -107,7 +107,8 @@ int mtj_xent(const float* logits, int64_t ld, const int32_t* target, int64_t M, 
 int mtj_gemm(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
              int dtype, int epi, void* out, int64_t ldo, int out_dtype, const mtj_inproj* ip, void* stream);
 
-/* mtj_gemm for skinny problems (M <= 64: batched decode): when the output has too few tiles to occupy the
+/* mtj_gemm for problems with few output tiles (batched decode; the out projection of a short prompt): when the
+ * output has too few tiles to occupy the
  * chip, K is cut into ranges that run as separate workgroups, each storing a float32 partial tile into `work`,
  * and a second kernel adds the partials in a fixed order (results do not depend on scheduling) and applies the
  * epilogue.  STORE and RESID only.  `work` holds mtj_gemm_splitk_work_bytes() bytes (0: no split is used and the

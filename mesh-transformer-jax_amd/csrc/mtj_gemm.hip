@@ -559,7 +559,7 @@ int dispatch_tile(const gemm_args& a, hipStream_t s) {
   if (a.M <= 64) return launch<T, EPI, 1, 4, 2, 2, BK, 2>(a, s);    // 64 x 256
   if constexpr (std::is_same<T, bf16_t>::value) {
     const int64_t big = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
-    if (big >= 200) return launch_dma<EPI>(a, s);                   // 256 x 256, 8 wavefronts of 128 x 64
+    if (big >= 200 && a.splits == 1) return launch_dma<EPI>(a, s);                   // 256 x 256, 8 wavefronts of 128 x 64
   }
   return launch<T, EPI, 2, 2, 2, 2, BK, 2>(a, s);                   // 128 x 128
 }
@@ -605,11 +605,17 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 
 // how many K ranges a skinny problem is cut into so that its few output tiles still fill the chip
 int pick_splits(int64_t M, int64_t N, int64_t K, int dtype) {
-  if (M > 64 || N % 4) return 1;
+  if (N % 4) return 1;
   const int bk = dtype == MTJ_BF16 ? 64 : 32;
-  const int64_t tiles = (N + 255) / 256, kt = K / bk;
+  const int64_t kt = K / bk;
   int splits = 1;
-  while (splits < 16 && tiles * splits * 2 <= 256 && kt % (splits * 2) == 0 && kt / (splits * 2) >= 4) splits *= 2;
+  if (M <= 64) {          // one row of 32/64 x 256 tiles: up to 16 ranges
+    const int64_t tiles = (N + 255) / 256;
+    while (splits < 16 && tiles * splits * 2 <= 256 && kt % (splits * 2) == 0 && kt / (splits * 2) >= 4) splits *= 2;
+  } else {                // 128 x 128 tiles, two workgroups per CU: up to 4 ranges (a short prompt's out projection)
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    while (splits < 4 && tiles * splits * 2 <= 512 && kt % (splits * 2) == 0 && kt / (splits * 2) >= 16) splits *= 2;
+  }
   return splits;
 }
 

@@ -129,6 +129,7 @@ class Session:
         self.q = torch.empty(B, H, dh, dtype=torch.float32, device=dev)
         self.logits = torch.empty(B, V, dtype=torch.float32, device=dev)
         nb = 0 if self.gemv_path else L.mtj_gemm_splitk_work_bytes(B, d, d + F, w.dtype)
+        nb = max(nb, L.mtj_gemm_splitk_work_bytes(M, d, d + F, w.dtype))     # the out projection of a short prefill
         self.gemm_work = torch.empty(max(nb, 256), dtype=torch.uint8, device=dev)
         self.attn_work = torch.zeros(max(L.mtj_attn_decode_work_bytes(B, H, dh, Tcap), 256), dtype=torch.uint8, device=dev)
         self.sample_work = None
@@ -203,8 +204,8 @@ class Engine:
                          None, 0, 0, C.byref(ip), s))
         check(L.mtj_attn_prefill(ptr(ses.q_pf), ptr(ses.kc[i]), ptr(ses.vt), ptr(pos0), ses.B, self.H, Tp, ses.Tcap,
                                  self.dh, ses.ldvt, ptr(act), d + F, w.dtype, ptr(key_limit), s))
-        check(L.mtj_gemm(ptr(act), d + F, ptr(w.w_out[i]), ptr(w.b2[i]), M, d, d + F, w.dtype, EPI_RESID,
-                         ptr(x), d, F32, None, s))
+        check(L.mtj_gemm_splitk(ptr(act), d + F, ptr(w.w_out[i]), ptr(w.b2[i]), M, d, d + F, w.dtype, EPI_RESID,
+                                ptr(x), d, F32, ptr(ses.gemm_work), ses.gemm_work.numel(), s))
 
     def embed_tok(self, ses):
         """x = EmbeddingShard(tok) for the decode step that follows."""

@@ -211,8 +211,6 @@ def main():
     ap.add_argument("--prefill-probe", action="store_true",
                     help="profiling probe: 6 forwards of one full-shape layer on 8 x 2048 tokens (BASELINE config 2) "
                          "on a 1-layer model of the 6B shape; prints the time per forward, no bench line")
-    ap.add_argument("--single-launch", type=int, default=None, choices=(0, 1),
-                    help="decode step as one persistent launch (1) or one launch per matrix (0); default: the library's")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the whole model on ONE GPU (no collectives, no sharding); "
@@ -238,8 +236,6 @@ def main():
         print(json.dumps({"layer_8x2048_ms": t * 1e3, "tflops": fl / t / 1e12, "frac_mfma": fl / t / 2.5e15}))
         return
     cfg = dict(CFG_6B, sampler=sampling.greedy_sample)
-    if args.single_launch is not None:
-        cfg["decode_single_launch"] = bool(args.single_launch)
     K, W = args.steps, args.warmup
     net = CausalTransformer(cfg, synthetic_tree(cfg, 2, dev, torch.bfloat16))
     P, L = 512, 2048

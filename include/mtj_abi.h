@@ -127,45 +127,6 @@ int mtj_gemv(const float* x, const float* ln_scale, const float* ln_offset, cons
              int64_t N, int64_t K, int dtype, int epi, void* out, int out_dtype, const mtj_inproj* ip,
              void* stream);
 
-/* One layer's operands for mtj_decode_step (device pointers; the array of these lives in device memory). */
-typedef struct {
-  const void* w_in;        /* [3d+F, d] packed q|v|k|fc_in          */
-  const void* w_out;       /* [d, d+F]  packed out|fc_out           */
-  const float* ln_scale;   /* [d]                                   */
-  const float* ln_offset;  /* [d]                                   */
-  const float* b1;         /* [F] fc_in bias                        */
-  const float* b2;         /* [d] fc_out bias                       */
-  void* k_cache;           /* [1, H, Tcap, dh] dtype, K rotated     */
-  void* v_cache;           /* [1, H, Tcap, dh]                      */
-} mtj_step_layer;
-
-/* A whole batch-1 decode step. */
-typedef struct {
-  const mtj_step_layer* layers;         /* device array [n_layers]                                        */
-  int32_t n_layers, d_model, n_heads, d_head, rotary_dims, Tcap, n_vocab, max_pos, dtype;
-  const int32_t* pos;                   /* [1] position of the token being decoded                        */
-  const float* sin_tab;                 /* [max_pos, r/2]                                                 */
-  const float* cos_tab;
-  float* x;                             /* [d] embedded token in, last residual out                       */
-  const float* pln_scale;               /* final LayerNorm and projection                                 */
-  const float* pln_offset;
-  const void* w_p;                      /* [V, d] packed                                                  */
-  const float* b_p;                     /* [V]                                                            */
-  float* logits;                        /* [V] out                                                        */
-} mtj_step;
-
-/* generate_once (transformer_shard.py:97-115) for a batch of one as ONE launch: all layers (LayerNorm, q|v|k|fc_in
- * with RoPE / K-V append / bias+GELU, attention over the window, out|fc_out + residual) and the final LayerNorm +
- * logits, by one resident workgroup per CU with grid barriers in between; arithmetic as in mtj_gemv / mtj_attn_decode.
- * `work`: mtj_decode_step_work_bytes() bytes, 256-byte aligned.  Its first 576 bytes are the barrier counters, which
- * the caller sets to zero before EVERY call (stream-ordered; with a fill kernel if the call is recorded into a graph);
- * the 32-bit word at byte 576 is a failure flag that the caller zeroes once and reads after synchronising.
- * The launch needs the whole GPU to itself: the workgroups wait for each other, and a workgroup that cannot become
- * resident makes the others give up after a bounded wait (the flag is then non-zero, stays so, and no logits are
- * valid).  No counterpart of the single launch exists in the reference (XLA schedules its own kernels). */
-int64_t mtj_decode_step_work_bytes(int64_t d_model, int64_t n_heads, int64_t d_head, int64_t Tcap);
-int mtj_decode_step(const mtj_step* step, void* work, void* stream);
-
 /* Causal self-attention over a left-padded rectangle (self_attn + masks of get_init_decode_state,
  * layers.py:260-285, 347-366).  q [B,H,Tp,dh], k_cache [B,H,Tcap,dh] (rotated), v_t [B,H,dh,ldvt] with
  * ldvt >= Tp rounded up to a multiple of 64 (columns beyond the last key may hold anything);

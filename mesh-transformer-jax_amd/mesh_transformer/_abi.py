@@ -33,24 +33,6 @@ class NextEmbed(C.Structure):
     _fields_ = [("w", _p), ("bias", _p), ("x_next", _p), ("d", _i64), ("dtype", C.c_int32)]
 
 
-class StepLayer(C.Structure):
-    """mtj_step_layer"""
-    _fields_ = [("w_in", _p), ("w_out", _p), ("ln_scale", _p), ("ln_offset", _p), ("b1", _p), ("b2", _p),
-                ("k_cache", _p), ("v_cache", _p)]
-
-
-class Step(C.Structure):
-    """mtj_step"""
-    _fields_ = [
-        ("layers", _p),
-        ("n_layers", C.c_int32), ("d_model", C.c_int32), ("n_heads", C.c_int32), ("d_head", C.c_int32),
-        ("rotary_dims", C.c_int32), ("Tcap", C.c_int32), ("n_vocab", C.c_int32), ("max_pos", C.c_int32),
-        ("dtype", C.c_int32),
-        ("pos", _p), ("sin_tab", _p), ("cos_tab", _p), ("x", _p), ("pln_scale", _p), ("pln_offset", _p),
-        ("w_p", _p), ("b_p", _p), ("logits", _p),
-    ]
-
-
 # name -> (restype, argtypes); one entry per declaration in mtj_abi.h
 SIGNATURES = {
     "mtj_version": (_i32, []),
@@ -63,8 +45,6 @@ SIGNATURES = {
     "mtj_gemm_splitk_work_bytes": (_i64, [_i64, _i64, _i64, _i32]),
     "mtj_gemm_splitk": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, _p, _i64, _p]),
     "mtj_gemv": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p, _i32, C.POINTER(InProj), _p]),
-    "mtj_decode_step_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),
-    "mtj_decode_step": (_i32, [C.POINTER(Step), _p, _p]),
     "mtj_attn_prefill": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64, _i32, _p, _p]),
     "mtj_attn_decode_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "mtj_attn_decode": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _i32, _i32, _p, _p]),

@@ -17,7 +17,7 @@ import numpy as np
 import torch
 
 from . import _abi
-from ._abi import BF16, EPI_INPROJ, EPI_RESID, EPI_STORE, F32, InProj, NextEmbed, Step, StepLayer, check, ptr
+from ._abi import BF16, EPI_INPROJ, EPI_RESID, EPI_STORE, F32, InProj, NextEmbed, check, ptr
 
 ROOT = "causal_transformer_shard/~/"
 
@@ -138,27 +138,6 @@ class Session:
         self.pos_start = torch.zeros(B, dtype=torch.int32, device=dev)
         self.pos0 = torch.zeros(B, dtype=torch.int32, device=dev)
         self.graphs = {}
-        # the whole decode step as one launch (batch 1 only): the description of the step and its work area
-        self.step = None
-        if self.gemv_path and eng.single_launch and w.w_p is not None:
-            arr = (StepLayer * len(w.layer_ids))()
-            for j, i in enumerate(w.layer_ids):
-                arr[j].w_in, arr[j].w_out = ptr(w.w_in[i]), ptr(w.w_out[i])
-                arr[j].ln_scale, arr[j].ln_offset = ptr(w.ln_s[i]), ptr(w.ln_o[i])
-                arr[j].b1, arr[j].b2 = ptr(w.b1[i]), ptr(w.b2[i])
-                arr[j].k_cache, arr[j].v_cache = ptr(self.kc[i]), ptr(self.vc[i])
-            self.step_layers = torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8).to(dev)
-            st = Step()
-            st.layers = ptr(self.step_layers)
-            st.n_layers, st.d_model, st.n_heads, st.d_head, st.rotary_dims = len(w.layer_ids), d, H, dh, eng.r
-            st.Tcap, st.n_vocab, st.max_pos, st.dtype = Tcap, V, max_pos, w.dtype
-            st.pos, st.sin_tab, st.cos_tab, st.x = ptr(self.pos), ptr(self.sin), ptr(self.cos), ptr(self.x)
-            st.pln_scale, st.pln_offset, st.w_p, st.b_p = ptr(w.pln_s), ptr(w.pln_o), ptr(w.w_p), ptr(w.b_p)
-            st.logits = ptr(self.logits)
-            self.step = st
-            self.step_work = torch.zeros(L.mtj_decode_step_work_bytes(d, H, dh, Tcap), dtype=torch.uint8, device=dev)
-            self.step_sync = self.step_work[:576].view(torch.int32)         # barrier counters, cleared before every step
-            self.step_fail = self.step_work[576:580].view(torch.int32)      # sticky: a barrier gave up waiting
 
 
 class Engine:
@@ -171,8 +150,6 @@ class Engine:
             raise NotImplementedError("only pe == 'rotary' is on the GPT-J path")
         self.config = config
         self.device = torch.device(device)
-        # batch-1 decode as one persistent launch per step instead of one launch per matrix / attention
-        self.single_launch = bool(config.get("decode_single_launch", False))
         self.H = config["n_heads"]
         d = config["d_model"]
         assert d % self.H == 0                                   # layers.py:238
@@ -249,10 +226,6 @@ class Engine:
         window is updated in place."""
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()
         B, d, F, V = ses.B, w.d, w.F, w.V
-        if ses.step is not None:
-            ses.step_sync.zero_()          # the barrier counters; a fill kernel, so the step can be recorded into a graph
-            check(L.mtj_decode_step(C.byref(ses.step), ptr(ses.step_work), s))
-            return
         for i in w.layer_ids:
             self.layer_decode(ses, i)
         if ses.gemv_path:
@@ -262,13 +235,6 @@ class Engine:
             check(L.mtj_layernorm(ptr(ses.x), ptr(w.pln_s), ptr(w.pln_o), B, d, ptr(ses.h), w.dtype, s))
             check(L.mtj_gemm(ptr(ses.h), d, ptr(w.w_p), ptr(w.b_p), B, V, d, w.dtype, EPI_STORE, ptr(ses.logits), V,
                              F32, None, s))
-
-    def check_step(self, ses):
-        """After a synchronisation: raises if a single-launch decode step gave up at a barrier."""
-        if ses.step is not None and int(ses.step_fail.item()) != 0:
-            ses.step_fail.zero_()
-            raise RuntimeError("mtj_decode_step: a workgroup waited too long at a grid barrier (the launch needs every "
-                               "compute unit of the GPU to itself); the generated tokens are not valid")
 
     def layer_decode(self, ses, i):
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()

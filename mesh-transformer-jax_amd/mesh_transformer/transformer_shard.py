@@ -184,7 +184,6 @@ class CausalTransformer:
                 timing.update(prefill_s=t1 - t0, prefill_tokens=B * Tp, warmup_s=t2 - t1, decode_s=t3 - t2,
                               decode_steps=G - W)
             torch.cuda.synchronize(dev)
-            eng.check_step(ses)
             toks = ses.out_tokens[:, :G].cpu().numpy().astype(np.uint32)[:, :, None]
             final_state = (toks[:, -1], ses, None)
             out = (toks, None)

@@ -53,7 +53,12 @@ struct gemv_args {
 // first, then the first U KiB of weights (so the LayerNorm prologue overlaps the first HBM round trip), and
 // every epilogue operand (position, sin/cos, biases, the residual) is fetched up front by the lane that
 // will finish that row - under load a dependent load costs tens of microseconds.
-template <typename T, int U>
+//
+// FULL: K is a whole number of wavefront tiles (U x 64 lanes x 16 bytes).  The rows of a wavefront are then one
+// contiguous run of whole tiles, which is streamed with two tiles in flight - the next one is requested before the
+// current one is consumed, so a wavefront never has an empty memory queue (a plain read of the same layout goes
+// from 6.8 to 7.7 TB/s with that) - and no load is conditional.
+template <typename T, int U, bool FULL>
 __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   extern __shared__ __align__(16) float xs[];
   __shared__ float red[2][16];
@@ -89,7 +94,11 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   }
   // ---- ... then the first tile of weights
   uint32x4 w[U];
-  if (nrows > 0) {
+  if (FULL) {
+    const T* rowp = W + (nrows > 0 ? row0 : 0) * a.K;      // a wavefront without rows reads (and drops) row 0
+#pragma unroll
+    for (int u = 0; u < U; ++u) w[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(rowp + u * STEP + lane * EPC));
+  } else if (nrows > 0) {
     const T* rowp = W + row0 * a.K;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -149,6 +158,45 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   // ---- stream my rows; lane r keeps the sum of row r
   const int tpr = (K + STEP * U - 1) / (STEP * U);          // tiles per row
   float mine = 0.f;
+  if (FULL) {
+    constexpr int TILE = STEP * U;
+    const T* base = W + row0 * a.K + lane * EPC;            // tile g of this wavefront starts at base + g * TILE
+    const int ntiles = nrows * tpr;
+    uint32x4 w2[U];
+    float acc = 0.f;
+    int kt = 0, r = 0;
+    auto consume = [&](const uint32x4 (&t)[U]) {
+      const float* xk = xs + kt * TILE + lane * EPC;
+#pragma unroll
+      for (int u = 0; u < U; ++u) chunk<T>::fma(t[u], xk + u * STEP, acc);
+      if (++kt == tpr) {                                    // the row is complete
+        const float sum = wave_sum(acc);
+        if (lane == r) mine = sum;
+        acc = 0.f; kt = 0; ++r;
+      }
+    };
+    auto request = [&](uint32x4 (&t)[U], int g) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        t[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(base + (int64_t)g * TILE + u * STEP));
+    };
+    // steady state without a conditional load: the wait before a tile is consumed then counts only the loads
+    // issued before it, and leaves the younger tile in flight
+    int g = 0;
+    for (; g + 2 < ntiles; g += 2) {
+      request(w2, g + 1);
+      consume(w);
+      request(w, g + 2);
+      consume(w2);
+    }
+    if (g + 1 < ntiles) {
+      request(w2, g + 1);
+      consume(w);
+      consume(w2);
+    } else if (g < ntiles) {
+      consume(w);
+    }
+  } else
   for (int r = 0; r < nrows; ++r) {
     const T* rowp = W + (row0 + r) * a.K;
     float acc = 0.f;
@@ -181,7 +229,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   }
 }
 
-template <typename T, int U>
+template <typename T, int U, bool FULL>
 int launch(const gemv_args& a, hipStream_t s) {
   const size_t lds = (size_t)a.K * sizeof(float);
   const int64_t units = a.epi == MTJ_EPI_INPROJ ? a.N / 2 : a.N;
@@ -192,18 +240,20 @@ int launch(const gemv_args& a, hipStream_t s) {
   while ((units + grid * 16 - 1) / (grid * 16) * upw > 62) grid *= 2;   // a lane per row: <= 64 rows per wavefront
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<T, U>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<T, U, FULL>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256);
     if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_gemv: hipFuncSetAttribute: %s", hipGetErrorString(e));
     attr_set = true;
   }
-  gemv_kernel<T, U><<<(unsigned)grid, 1024, lds, s>>>(a);
+  gemv_kernel<T, U, FULL><<<(unsigned)grid, 1024, lds, s>>>(a);
   return mtj_check_launch("mtj_gemv");
 }
 
 template <typename T>
 int dispatch(const gemv_args& a, hipStream_t s) {
-  return launch<T, 8>(a, s);
+  constexpr int U = 8;
+  if (a.K % (U * 64 * chunk<T>::EPC) == 0) return launch<T, U, true>(a, s);
+  return launch<T, U, false>(a, s);
 }
 
 }  // namespace

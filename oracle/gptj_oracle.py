@@ -114,6 +114,38 @@ def seeded_params(cfg, seed: int, weight_dtype=torch.float32, std: float = 0.02)
     return out
 
 
+def hashed_params(cfg, seed: int, weight_dtype=torch.bfloat16, std: float = 0.02, device="cpu"):
+    """Synthetic tree for sizes where drawing normals on the host is too slow and a device generator would not be
+    reproducible elsewhere: element i of leaf number j (sorted key order) is a 16-bit integer hash of (seed, j, i),
+    centred and scaled to standard deviation `std` (uniform, not normal).  Integer arithmetic, one exact
+    subtraction and one float32 multiplication: the same bits on any device.  LayerNorm scale = 1, offset = 0."""
+    shapes = param_shapes(cfg)
+    scale = np.float32(std * np.sqrt(12.0) / 65536.0)
+    out, j = {}, 0
+    for mod in sorted(shapes):
+        out[mod] = {}
+        for leaf in sorted(shapes[mod]):
+            shp = shapes[mod][leaf]
+            j += 1
+            if leaf == "scale":
+                a = torch.ones(shp, dtype=torch.float32, device=device)
+            elif leaf == "offset":
+                a = torch.zeros(shp, dtype=torch.float32, device=device)
+            else:
+                n = int(np.prod(shp))
+                h = torch.arange(n, dtype=torch.int64, device=device)
+                h = (h * 2654435761 + (seed * 1000003 + j) * 40503) & 0xFFFFFFFF
+                h ^= h >> 15
+                h = (h * 2246822519) & 0xFFFFFFFF
+                h ^= h >> 13
+                h = (h * 3266489917) & 0xFFFFFFFF
+                h ^= h >> 16
+                a = (((h & 0xFFFF).to(torch.float32) - 32767.5) * float(scale)).reshape(shp)
+                del h
+            out[mod][leaf] = a.to(weight_dtype)
+    return out
+
+
 def seeded_prompt(seed: int, batch: int, n: int, hi: int = 50257) -> np.ndarray:
     rng = np.random.Generator(np.random.Philox(seed + 1000003))
     return rng.integers(0, hi, size=(batch, n), dtype=np.int64).astype(np.uint32)

@@ -1,7 +1,7 @@
 """Size-independent properties at the full GPT-J-6B shapes (28 layers, d_model 4096, 16 heads x 256, vocab 50400,
-bf16 random-init weights): the CPU oracle cannot run these sizes in reasonable time, so the checks here are
+bf16 random-init weights): the CPU oracle takes minutes and tens of GB at these sizes, so most checks here are
 relations that must hold whatever the weights are, between code paths that are each compared with the oracle at
-small sizes elsewhere."""
+small sizes elsewhere; one short decode run of the oracle itself at this shape is committed as a fixture."""
 import numpy as np
 import pytest
 import torch
@@ -103,3 +103,30 @@ def test_batch32_nucleus_decode_rows_are_independent(net6b):
     same = (out2[0][:, :, 0] == toks[[0, 4]]).mean()
     print("fraction of tokens reproduced at batch 2:", same)
     assert same > 0.5      # other tile shapes round differently; a flat random-init distribution amplifies that
+
+
+def test_decode_against_the_committed_6b_oracle_run():
+    """The CPU oracle's own run at the full 6B shape (tests/golden/gptj6b_decode.npz, written by
+    tests/golden/make_golden_6b.py: float32 arithmetic on the bf16 hashed synthetic tree, 128-token prompt, 8 greedy
+    steps): |dlogit| <= 2e-2 on every stored logit and the same greedy tokens."""
+    import os
+    from oracle import gptj_oracle as O
+    from mesh_transformer import sampling
+    from mesh_transformer.transformer_shard import CausalTransformer
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gptj6b_decode.npz"))
+    dev = torch.device("cuda:0")
+    tree = O.hashed_params(CFG_6B, int(g["seed"]), torch.bfloat16, device=dev)
+    net = CausalTransformer(dict(CFG_6B, sampler=sampling.greedy_sample), tree)
+    prompt = g["prompt"]
+    G = len(g["tokens"])
+    _, out = net.generate(prompt, [prompt.shape[1]], G, {}, return_logits=True)
+    lg = out[2][0, :, 0]                                            # [G, V]
+    stride = int(g["stride"])
+    e1 = np.abs(lg[:, ::stride] - g["strided_logits"]).max()
+    e2 = np.abs(np.take_along_axis(lg, g["top_ids"].astype(np.int64), -1) - g["top_logits"]).max()
+    print("6B decode vs the oracle's run: max |dlogit| strided", e1, "top-32", e2)
+    assert e1 < 2e-2 and e2 < 2e-2
+    assert np.abs(lg.astype(np.float64).sum(-1) - g["logit_sum"]).max() < 2e-2 * lg.shape[1] ** 0.5 * 4
+    assert np.array_equal(out[0][0, :, 0].astype(np.int64), g["tokens"])
+    del net, tree
+    torch.cuda.empty_cache()

@@ -197,7 +197,9 @@ def test_gemm_rejects_bad_arguments(L):
 
 # ------------------------------------------------------------------ GEMV
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
-@pytest.mark.parametrize("N,K", [(512, 256), (28672, 4096), (4096, 20480), (50400, 4096), (514, 2560), (6, 520)])
+@pytest.mark.parametrize("N,K", [(512, 256), (28672, 4096), (4096, 20480), (50400, 4096), (514, 2560), (6, 520),
+                                 # whole-tile rows with 0 or 1, exactly 1, 3, and 4-or-5 tiles per wavefront
+                                 (8, 4096), (4096, 4096), (12288, 4096), (9000, 8192)])
 def test_gemv_store_resid_and_layernorm(L, dt, N, K):
     a = abi()
     g = torch.Generator().manual_seed(N + K)

@@ -441,12 +441,16 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
   const int voff_a = (int)((int64_t)lr * a.lda * 2) + lc, voff_b = (int)((int64_t)lr * a.K * 2) + lc;
   const int pass_a = (int)((int64_t)ROWS_PER_LOAD * a.lda * 2), pass_b = (int)((int64_t)ROWS_PER_LOAD * a.K * 2);
 
-  // load number l of a k-tile: l < LOADS fetches rows [l*64, l*64+64) of A, the others of W
+  // my K range (split-K: blockIdx.y; the whole of K otherwise), in k-tiles
+  const int kt0 = (int)((int64_t)blockIdx.y * (a.K / BK) / a.splits);
+  const int KT = (int)((int64_t)(blockIdx.y + 1) * (a.K / BK) / a.splits) - kt0;
+
+  // load number l of k-tile kt of my range: l < LOADS fetches rows [l*64, l*64+64) of A, the others of W
   auto issue_one = [&](int st, int kt, auto L_) {
     constexpr int l = decltype(L_)::value, part = l / LOADS, i = l % LOADS;
     unsigned char* dst = smem + st * STAGEB + part * OPB + i * (NT * 16) + wave_s * 1024;
-    if (part == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr)dst, 16, voff_a, kt * ROWB + i * pass_a, 0, 0);
-    else __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr)dst, 16, voff_b, kt * ROWB + i * pass_b, 0, 0);
+    if (part == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr)dst, 16, voff_a, (kt0 + kt) * ROWB + i * pass_a, 0, 0);
+    else __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr)dst, 16, voff_b, (kt0 + kt) * ROWB + i * pass_b, 0, 0);
   };
 
   floatx16 acc[WM][WN];
@@ -457,7 +461,6 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  const int KT = a.K / BK;
   for_stages<0, 2 * LOADS>([&](auto L_) { issue_one(0, 0, L_); });
   if (KT > 1) for_stages<0, 2 * LOADS>([&](auto L_) { issue_one(1, 1, L_); });
 
@@ -517,7 +520,8 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
       if (kt + decltype(S_)::value < KT) k_tile(kt + decltype(S_)::value, S_);
     });
 
-  epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, a.out, acc, smem, m0, n0);
+  void* out = a.splits > 1 ? (void*)(reinterpret_cast<float*>(a.out) + blockIdx.y * a.split_stride) : a.out;
+  epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, out, acc, smem, m0, n0);
 }
 
 template <int EPI>
@@ -531,7 +535,7 @@ int launch_dma(const gemm_args& a, hipStream_t s) {
     attr_set = true;
   }
   const int tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
-  gemm_dma_kernel<EPI><<<tiles, 512, lds, s>>>(a);
+  gemm_dma_kernel<EPI><<<dim3(tiles, a.splits), 512, lds, s>>>(a);
   return mtj_check_launch("mtj_gemm");
 }
 
@@ -559,7 +563,7 @@ int dispatch_tile(const gemm_args& a, hipStream_t s) {
   if (a.M <= 64) return launch<T, EPI, 1, 4, 2, 2, BK, 2>(a, s);    // 64 x 256
   if constexpr (std::is_same<T, bf16_t>::value) {
     const int64_t big = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
-    if (big >= 200 && a.splits == 1) return launch_dma<EPI>(a, s);                   // 256 x 256, 8 wavefronts of 128 x 64
+    if (big * a.splits >= 200) return launch_dma<EPI>(a, s);                         // 256 x 256, 8 wavefronts of 128 x 64
   }
   return launch<T, EPI, 2, 2, 2, 2, BK, 2>(a, s);                   // 128 x 128
 }
@@ -612,7 +616,14 @@ int pick_splits(int64_t M, int64_t N, int64_t K, int dtype) {
   if (M <= 64) {          // one row of 32/64 x 256 tiles: up to 16 ranges
     const int64_t tiles = (N + 255) / 256;
     while (splits < 16 && tiles * splits * 2 <= 256 && kt % (splits * 2) == 0 && kt / (splits * 2) >= 4) splits *= 2;
-  } else {                // 128 x 128 tiles, two workgroups per CU: up to 4 ranges (a short prompt's out projection)
+  } else {
+    if (dtype == MTJ_BF16) {   // 256 x 256 tiles of the direct-to-LDS kernel, one workgroup per CU (a short prompt's out projection)
+      const int64_t big = ((M + 255) / 256) * ((N + 255) / 256);
+      while (splits < 16 && big * splits * 2 <= 256 && kt % (splits * 2) == 0 && kt / (splits * 2) >= 16) splits *= 2;
+      if (big * splits >= 200) return splits;
+      splits = 1;
+    }
+    // 128 x 128 tiles, two workgroups per CU: up to 4 ranges
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
     while (splits < 4 && tiles * splits * 2 <= 512 && kt % (splits * 2) == 0 && kt / (splits * 2) >= 16) splits *= 2;
   }

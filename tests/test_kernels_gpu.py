@@ -150,7 +150,7 @@ def test_gemm_store_and_resid(L, dt, M, N, K):
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("M,N,K", [(32, 4096, 20480), (5, 512, 2560), (64, 260, 1024), (8, 50400, 4096), (3, 64, 64),
-                                   (511, 4096, 20480), (200, 512, 2560), (700, 1024, 4096)])
+                                   (511, 4096, 20480), (200, 512, 2560), (700, 1024, 4096), (130, 4096, 20480), (300, 2048, 8192)])
 def test_gemm_splitk_matches_reference_and_is_deterministic(L, dt, M, N, K):
     """Skinny products: K ranges run as separate workgroups and are added in a fixed order."""
     a = abi()

@@ -56,8 +56,9 @@ struct gemv_args {
 //
 // FULL: K is a whole number of wavefront tiles (U x 64 lanes x 16 bytes).  The rows of a wavefront are then one
 // contiguous run of whole tiles, which is streamed with two tiles in flight - the next one is requested before the
-// current one is consumed, so a wavefront never has an empty memory queue (a plain read of the same layout goes
-// from 6.8 to 7.7 TB/s with that) - and no load is conditional.
+// current one is consumed, so a wavefront never has an empty memory queue - and no load is conditional.  (Dealing
+// the rows out round-robin instead, so that the chip reads one contiguous window at a time, streams ~5 % faster in
+// a plain read but scatters every lane's epilogue loads and stores: 43.5 us against 40.2 for the 235 MB launch.)
 template <typename T, int U, bool FULL>
 __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   extern __shared__ __align__(16) float xs[];

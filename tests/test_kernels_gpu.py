@@ -391,7 +391,9 @@ def test_attn_prefill(L, dt, dh, H, Tp):
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("dh,H", [(64, 8), (256, 16)])
-@pytest.mark.parametrize("Tcap,positions", [(7, [0, 6, 9]), (300, [0, 150, 299]), (2047, [511, 2046, 5000])])
+@pytest.mark.parametrize("Tcap,positions", [(7, [0, 6, 9]), (300, [0, 150, 299]), (2047, [511, 2046, 5000]),
+                                            # many sequences, ragged positions, some beyond the window
+                                            (1000, [(i * 131) % 1300 for i in range(24)])])
 def test_attn_decode_window(L, dt, dh, H, Tcap, positions):
     a = abi()
     g = torch.Generator().manual_seed(Tcap + dh)

@@ -307,7 +307,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
       ra[st][i] = __builtin_amdgcn_raw_buffer_load_b128(ra_rsrc, voff_a, koff + i * pass_a, 0);
 #pragma unroll
     for (int i = 0; i < B_CHUNKS; ++i)
-      rb[st][i] = __builtin_amdgcn_raw_buffer_load_b128(rb_rsrc, voff_b, koff + i * pass_b, 0);
+      rb[st][i] = __builtin_amdgcn_raw_buffer_load_b128(rb_rsrc, voff_b, koff + i * pass_b, BM <= 64 ? 2 : 0);  // nt: streamed once
   };
   auto store_lds = [&](auto ST_, int buf) {
     constexpr int st = decltype(ST_)::value;
@@ -337,8 +337,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
   if (NS < KT) load_global(std::integral_constant<int, 0>{}, NS);
   __syncthreads();
 
-  // one k-tile; PARK = stage of k-tile kt+1 (a compile-time index: the k loop is unrolled by NS)
-  auto k_tile = [&](int kt, auto PARK_) {
+  // one k-tile; PARK = stage of k-tile kt+1 (a compile-time index: the k loop is unrolled by NS).  STEADY: k-tiles
+  // kt+1 and kt+1+NS both exist, so the park and the request are unconditional.  That matters: the wait the
+  // compiler puts before the park is the strictest over all paths that reach it, and with the request under a
+  // condition that is "everything outstanding", the request of one iteration ago included.
+  auto k_tile = [&](int kt, auto PARK_, auto STEADY_) {
+    constexpr bool steady = decltype(STEADY_)::value;
     const int buf = kt & 1;
     const T* as = As + (buf * BM + wm * WM * 32 + fr) * LDS_ROW + fg * 8;
     const T* bs = Bs + (buf * BN + wn * WN * 32 + fr) * LDS_ROW + fg * 8;
@@ -364,16 +368,21 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
         for (int j = 0; j < WN; ++j) mma<T>::run(acc[i][j], fa[cur][i], fb[cur][j]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (kt + 1 < KT) store_lds(PARK_, buf ^ 1);
-    if (kt + 1 + NS < KT) load_global(PARK_, kt + 1 + NS);
+    if (steady || kt + 1 < KT) store_lds(PARK_, buf ^ 1);
+    if (steady || kt + 1 + NS < KT) load_global(PARK_, kt + 1 + NS);
     __syncthreads();
   };
-  for (int kt = 0; kt < KT; kt += NS) {
+  int kt = 0;
+  for (; kt + 2 * NS < KT; kt += NS)          // the last k-tile of the round, kt+NS-1, still requests kt+2*NS
     for_stages<0, NS>([&](auto S_) {
       constexpr int s = decltype(S_)::value;
-      if (kt + s < KT) k_tile(kt + s, std::integral_constant<int, (s + 1) % NS>{});
+      k_tile(kt + s, std::integral_constant<int, (s + 1) % NS>{}, std::true_type{});
     });
-  }
+  for (; kt < KT; kt += NS)
+    for_stages<0, NS>([&](auto S_) {
+      constexpr int s = decltype(S_)::value;
+      if (kt + s < KT) k_tile(kt + s, std::integral_constant<int, (s + 1) % NS>{}, std::false_type{});
+    });
 
   void* out = a.splits > 1 ? (void*)(reinterpret_cast<float*>(a.out) + blockIdx.y * a.split_stride) : a.out;
   epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, out, acc, smem, m0, n0);
@@ -559,8 +568,8 @@ int launch(const gemm_args& a, hipStream_t s) {
 
 template <typename T, int EPI, int BK>
 int dispatch_tile(const gemm_args& a, hipStream_t s) {
-  if (a.M <= 32) return launch<T, EPI, 1, 4, 1, 2, BK, 2>(a, s);    // 32 x 256: batched decode, weights stream once
-  if (a.M <= 64) return launch<T, EPI, 1, 4, 2, 2, BK, 2>(a, s);    // 64 x 256
+  if (a.M <= 32) return launch<T, EPI, 1, 4, 1, 1, BK, 2>(a, s);    // 32 x 128: batched decode, weights stream once
+  if (a.M <= 64) return launch<T, EPI, 1, 4, 2, 1, BK, 2>(a, s);    // 64 x 128
   if constexpr (std::is_same<T, bf16_t>::value) {
     const int64_t big = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
     if (big * a.splits >= 200) return launch_dma<EPI>(a, s);                         // 256 x 256, 8 wavefronts of 128 x 64
@@ -613,8 +622,8 @@ int pick_splits(int64_t M, int64_t N, int64_t K, int dtype) {
   const int bk = dtype == MTJ_BF16 ? 64 : 32;
   const int64_t kt = K / bk;
   int splits = 1;
-  if (M <= 64) {          // one row of 32/64 x 256 tiles: up to 16 ranges
-    const int64_t tiles = (N + 255) / 256;
+  if (M <= 64) {          // one row of 32 x 128 or 64 x 128 tiles: up to 16 ranges
+    const int64_t tiles = (N + 127) / 128;
     while (splits < 16 && tiles * splits * 2 <= 256 && kt % (splits * 2) == 0 && kt / (splits * 2) >= 4) splits *= 2;
   } else {
     if (dtype == MTJ_BF16) {   // 256 x 256 tiles of the direct-to-LDS kernel, one workgroup per CU (a short prompt's out projection)

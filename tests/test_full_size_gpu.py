@@ -91,18 +91,23 @@ def test_batch32_nucleus_decode_rows_are_independent(net6b):
     ctx[:, L - P:] = ids
     opts = {"top_p": np.full(B, 0.9), "temp": np.full(B, 0.8)}
     tm = {"warmup": 9}
-    _, out = net6b.generate(ctx, np.full(B, P), G, opts, uniforms=u, timing=tm)
+    _, out = net6b.generate(ctx, np.full(B, P), G, opts, uniforms=u, timing=tm, return_logits=True)
     toks = out[0][:, :, 0]
     print(f"batch-32 nucleus decode: {tm['decode_s'] / tm['decode_steps'] * 1e3:.3f} ms/step, "
           f"{B * tm['decode_steps'] / tm['decode_s']:.0f} tok/s")
     assert toks.shape == (B, G) and toks.max() < 50400
     assert np.array_equal(toks[0], toks[17])
     assert not np.array_equal(toks[4], toks[9])           # same prompt, different uniforms
-    # the same two rows alone (batch 2, still the batched kernels) reproduce their streams
-    _, out2 = net6b.generate(ctx[[0, 4]], [P, P], G, {"top_p": np.full(2, 0.9), "temp": np.full(2, 0.8)}, uniforms=u[[0, 4]])
-    same = (out2[0][:, :, 0] == toks[[0, 4]]).mean()
-    print("fraction of tokens reproduced at batch 2:", same)
-    assert same > 0.5      # other tile shapes round differently; a flat random-init distribution amplifies that
+    # The same two rows alone (batch 2, still the batched kernels, other tile shapes and K ranges in the prefill):
+    # the logits of the first step, whose inputs are the prompt alone, agree as two paths that are each within
+    # 2e-2 of the exact result do.  (The sampled
+    # streams need not: with a flat random-init distribution the nucleus holds thousands of tokens and a logit
+    # change of 1e-3 moves the inverse-CDF draw to a neighbour.)
+    _, out2 = net6b.generate(ctx[[0, 4]], [P, P], 2, {"top_p": np.full(2, 0.9), "temp": np.full(2, 0.8)},
+                             uniforms=u[[0, 4], :2], return_logits=True)
+    d = np.abs(out2[2][:, 0, 0] - out[2][[0, 4], 0, 0]).max()
+    print("first-step logits, batch 2 against batch 32: max |d|", d)
+    assert d < 4e-2
 
 
 def test_decode_against_the_committed_6b_oracle_run():

@@ -119,6 +119,14 @@ int mtj_gemm_splitk(const void* A, int64_t lda, const void* W, const float* bias
                     int dtype, int epi, void* out, int64_t ldo, int out_dtype, void* work, int64_t work_bytes,
                     void* stream);
 
+/* mtj_gemm_splitk with the RESID epilogue, followed in the same launch by the LayerNorm of the rows it completes:
+ * x [M, ldx] float32 += A x W^T + bias, then h [M, ldh] (h_dtype) = ReplicatedLayerNorm(x) with ln_scale / ln_offset
+ * [N] (layers.py:17-36) - the LayerNorm of the next layer, or of the projection, that follows the residual add in
+ * generate_once (transformer_shard.py:97-115).  `work` as for mtj_gemm_splitk; N <= 16384. */
+int mtj_gemm_splitk_ln(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
+                       int dtype, float* x, int64_t ldx, void* work, int64_t work_bytes, const float* ln_scale,
+                       const float* ln_offset, void* h, int64_t ldh, int h_dtype, void* stream);
+
 /* Batch-1 decode matrix-vector product: y = f(x) @ W^T with float32 activations and float32 accumulation
  * (jnp.dot(f32, bf16) semantics of hk.Linear at decode, layers.py:316-344).  x float32 [K].
  * If ln_scale != NULL the kernel first applies LayerNorm(x) (layers.py:17-36) - x then has K = d entries.

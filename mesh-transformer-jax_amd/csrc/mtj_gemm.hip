@@ -616,6 +616,87 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   }
 }
 
+// The RESID reduce of one whole row per workgroup, followed by the LayerNorm of the row it has just completed
+// (ReplicatedLayerNorm, layers.py:17-36, of the NEXT layer or of the projection): x += sum of partials + bias, then
+// h = scale * (x - mean) * rsqrt(var + 1e-5) + offset in h_dtype.  Saves the LayerNorm launch and its round trip
+// through memory between two decode layers.  N <= 4 * RLN_Q * 1024.
+constexpr int RLN_Q = 4;
+__global__ __launch_bounds__(1024) void splitk_reduce_ln_kernel(const float* __restrict__ work, int splits,
+                                                                int64_t split_stride, int N, const float* __restrict__ bias,
+                                                                float* __restrict__ x, int64_t ldx,
+                                                                const float* __restrict__ ln_scale,
+                                                                const float* __restrict__ ln_offset, void* __restrict__ h,
+                                                                int64_t ldh, int h_dtype) {
+  __shared__ float red[2][16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = blockIdx.x, nq = N / 4;
+  floatx4 v[RLN_Q];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < RLN_Q; ++i) {
+    const int q = i * 1024 + tid;
+    if (q < nq) {
+      const int n = q * 4;
+      floatx4 acc = *reinterpret_cast<const floatx4*>(work + (int64_t)m * N + n);
+      for (int sp = 1; sp < splits; ++sp) {
+        const floatx4 p = *reinterpret_cast<const floatx4*>(work + sp * split_stride + (int64_t)m * N + n);
+        acc.x += p.x; acc.y += p.y; acc.z += p.z; acc.w += p.w;
+      }
+      if (bias) {
+        const floatx4 b = *reinterpret_cast<const floatx4*>(bias + n);
+        acc.x += b.x; acc.y += b.y; acc.z += b.z; acc.w += b.w;
+      }
+      float* o = x + (int64_t)m * ldx + n;
+      const floatx4 old = *reinterpret_cast<const floatx4*>(o);
+      // the same two roundings per element as "o[j] += acc.j" of the plain reduce
+      acc.x = old.x + acc.x; acc.y = old.y + acc.y; acc.z = old.z + acc.z; acc.w = old.w + acc.w;
+      *reinterpret_cast<floatx4*>(o) = acc;
+      v[i] = acc;
+      sum += (acc.x + acc.y) + (acc.z + acc.w);
+    }
+  }
+  sum = wave_sum(sum);
+  if (lane == 0) red[0][wave] = sum;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) tot += red[0][i];
+  const float mean = tot / (float)N;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < RLN_Q; ++i) {
+    if (i * 1024 + tid < nq) {
+      const floatx4 t = v[i] - mean;
+      sq += (t.x * t.x + t.y * t.y) + (t.z * t.z + t.w * t.w);
+    }
+  }
+  sq = wave_sum(sq);
+  if (lane == 0) red[1][wave] = sq;
+  __syncthreads();
+  float var = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) var += red[1][i];
+  const float inv = rsqrtf(var / (float)N + 1e-5f);
+#pragma unroll
+  for (int i = 0; i < RLN_Q; ++i) {
+    const int q = i * 1024 + tid;
+    if (q < nq) {
+      const int n = q * 4;
+      const floatx4 sc = *reinterpret_cast<const floatx4*>(ln_scale + n);
+      const floatx4 of = *reinterpret_cast<const floatx4*>(ln_offset + n);
+      const floatx4 y = (sc * inv) * (v[i] - mean) + of;
+      if (h_dtype == MTJ_F32) {
+        *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(h) + (int64_t)m * ldh + n) = y;
+      } else {
+        uint32x2 pk;
+        pk.x = pack_bf16x2(y.x, y.y);
+        pk.y = pack_bf16x2(y.z, y.w);
+        *reinterpret_cast<uint32x2*>(reinterpret_cast<uint16_t*>(h) + (int64_t)m * ldh + n) = pk;
+      }
+    }
+  }
+}
+
 // how many K ranges a skinny problem is cut into so that its few output tiles still fill the chip
 int pick_splits(int64_t M, int64_t N, int64_t K, int dtype) {
   if (N % 4) return 1;
@@ -722,4 +803,35 @@ extern "C" int mtj_gemm_splitk(const void* A, int64_t lda, const void* W, const 
   else
     splitk_reduce_kernel<MTJ_EPI_STORE><<<grid, 256, 0, s>>>((const float*)work, splits, M * N, (int)M, (int)N, bias, out, ldo, out_dtype);
   return mtj_check_launch("mtj_gemm_splitk");
+}
+
+extern "C" int mtj_gemm_splitk_ln(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N,
+                                  int64_t K, int dtype, float* x, int64_t ldx, void* work, int64_t work_bytes,
+                                  const float* ln_scale, const float* ln_offset, void* h, int64_t ldh, int h_dtype,
+                                  void* stream) {
+  MTJ_REQUIRE(ln_scale && ln_offset && h && x, MTJ_EINVAL, "mtj_gemm_splitk_ln: null pointer");
+  MTJ_REQUIRE(h_dtype == MTJ_F32 || h_dtype == MTJ_BF16, MTJ_EDTYPE, "mtj_gemm_splitk_ln: h_dtype %d", h_dtype);
+  MTJ_REQUIRE(N % 4 == 0 && N <= 4 * RLN_Q * 1024 && ldh >= N && ldh % 4 == 0 && ldx >= N && ldx % 4 == 0 &&
+                  mtj_aligned16(x) && mtj_aligned16(h) && mtj_aligned16(ln_scale) && mtj_aligned16(ln_offset) &&
+                  (!bias || mtj_aligned16(bias)),
+              MTJ_EINVAL, "mtj_gemm_splitk_ln: N a multiple of 4 and <= %d, rows of x and h 16-byte aligned", 4 * RLN_Q * 1024);
+  if (int rc = check_common(A, lda, W, M, N, K, dtype, "mtj_gemm_splitk_ln")) return rc;
+  const int splits = pick_splits(M, N, K, dtype);
+  hipStream_t s = (hipStream_t)stream;
+  if (splits == 1) {      // no partials to reduce: the product with its own residual epilogue, then the plain LayerNorm
+    if (int rc = mtj_gemm(A, lda, W, bias, M, N, K, dtype, MTJ_EPI_RESID, x, ldx, MTJ_F32, nullptr, stream)) return rc;
+    MTJ_REQUIRE(ldx == N && ldh == N, MTJ_EINVAL, "mtj_gemm_splitk_ln: without a split, x and h must be dense");
+    return mtj_layernorm(x, ln_scale, ln_offset, M, N, h, h_dtype, stream);
+  }
+  MTJ_REQUIRE(work && mtj_aligned16(work) && work_bytes >= (int64_t)splits * M * N * (int64_t)sizeof(float), MTJ_EINVAL,
+              "mtj_gemm_splitk_ln: work must hold mtj_gemm_splitk_work_bytes() bytes");
+  gemm_args a{};
+  a.A = A; a.lda = lda; a.W = W; a.bias = nullptr; a.M = (int)M; a.N = (int)N; a.K = (int)K;
+  a.out = work; a.ldo = N; a.out_dtype = MTJ_F32; a.kv_dtype = dtype;
+  a.splits = splits; a.split_stride = M * N;
+  const int rc = dtype == MTJ_BF16 ? dispatch<bf16_t, 64>(a, MTJ_EPI_STORE, s) : dispatch<float, 32>(a, MTJ_EPI_STORE, s);
+  if (rc) return rc;
+  splitk_reduce_ln_kernel<<<(unsigned)M, 1024, 0, s>>>((const float*)work, splits, M * N, (int)N, bias, x, ldx, ln_scale,
+                                                       ln_offset, h, ldh, h_dtype);
+  return mtj_check_launch("mtj_gemm_splitk_ln");
 }

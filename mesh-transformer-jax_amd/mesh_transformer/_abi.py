@@ -44,6 +44,7 @@ SIGNATURES = {
     "mtj_gemm": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, C.POINTER(InProj), _p]),
     "mtj_gemm_splitk_work_bytes": (_i64, [_i64, _i64, _i64, _i32]),
     "mtj_gemm_splitk": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, _p, _i64, _p]),
+    "mtj_gemm_splitk_ln": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _p, _i64, _p, _i64, _p, _p, _p, _i64, _i32, _p]),
     "mtj_gemv": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p, _i32, C.POINTER(InProj), _p]),
     "mtj_attn_prefill": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64, _i32, _p, _p]),
     "mtj_attn_decode_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),

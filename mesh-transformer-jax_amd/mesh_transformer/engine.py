@@ -226,6 +226,17 @@ class Engine:
         window is updated in place."""
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()
         B, d, F, V = ses.B, w.d, w.F, w.V
+        if not ses.gemv_path and w.w_p is not None:
+            # batched decode: the reduce of every out projection also applies the LayerNorm that follows it (the
+            # next layer's, at the end the projection's), so only the first layer launches a LayerNorm of its own
+            ids = w.layer_ids
+            check(L.mtj_layernorm(ptr(ses.x), ptr(w.ln_s[ids[0]]), ptr(w.ln_o[ids[0]]), B, d, ptr(ses.h), w.dtype, s))
+            for j, i in enumerate(ids):
+                nxt = (w.ln_s[ids[j + 1]], w.ln_o[ids[j + 1]]) if j + 1 < len(ids) else (w.pln_s, w.pln_o)
+                self.layer_decode(ses, i, normed=True, next_ln=nxt)
+            check(L.mtj_gemm(ptr(ses.h), d, ptr(w.w_p), ptr(w.b_p), B, V, d, w.dtype, EPI_STORE, ptr(ses.logits), V,
+                             F32, None, s))
+            return
         for i in w.layer_ids:
             self.layer_decode(ses, i)
         if ses.gemv_path:
@@ -236,7 +247,9 @@ class Engine:
             check(L.mtj_gemm(ptr(ses.h), d, ptr(w.w_p), ptr(w.b_p), B, V, d, w.dtype, EPI_STORE, ptr(ses.logits), V,
                              F32, None, s))
 
-    def layer_decode(self, ses, i):
+    def layer_decode(self, ses, i, normed=False, next_ln=None):
+        """decode_once of layer i plus the residual add.  normed: ses.h already holds LayerNorm_i(ses.x); next_ln:
+        (scale, offset) of the LayerNorm that follows the residual add, applied into ses.h by the same launch."""
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()
         B, d, F = ses.B, w.d, w.F
         if ses.gemv_path:
@@ -248,14 +261,20 @@ class Engine:
             check(L.mtj_gemv(ptr(ses.act), None, None, ptr(w.w_out[i]), ptr(w.b2[i]), d, d + F, w.dtype, EPI_RESID,
                              ptr(ses.x), F32, None, s))
         else:
-            check(L.mtj_layernorm(ptr(ses.x), ptr(w.ln_s[i]), ptr(w.ln_o[i]), B, d, ptr(ses.h), w.dtype, s))
+            if not normed:
+                check(L.mtj_layernorm(ptr(ses.x), ptr(w.ln_s[i]), ptr(w.ln_o[i]), B, d, ptr(ses.h), w.dtype, s))
             ip = self._inproj(ses, i, 1, ses.pos, ses.q, F32, ses.act, w.dtype, None)
             check(L.mtj_gemm(ptr(ses.h), d, ptr(w.w_in[i]), ptr(w.b1[i]), B, 3 * d + F, d, w.dtype, EPI_INPROJ,
                              None, 0, 0, C.byref(ip), s))
             check(L.mtj_attn_decode(ptr(ses.q), ptr(ses.kc[i]), ptr(ses.vc[i]), ptr(ses.pos), B, self.H, ses.Tcap,
                                     self.dh, ptr(ses.act), d + F, w.dtype, w.dtype, ptr(ses.attn_work), s))
-            check(L.mtj_gemm_splitk(ptr(ses.act), d + F, ptr(w.w_out[i]), ptr(w.b2[i]), B, d, d + F, w.dtype, EPI_RESID,
-                                    ptr(ses.x), d, F32, ptr(ses.gemm_work), ses.gemm_work.numel(), s))
+            if next_ln is not None:
+                check(L.mtj_gemm_splitk_ln(ptr(ses.act), d + F, ptr(w.w_out[i]), ptr(w.b2[i]), B, d, d + F, w.dtype,
+                                           ptr(ses.x), d, ptr(ses.gemm_work), ses.gemm_work.numel(), ptr(next_ln[0]),
+                                           ptr(next_ln[1]), ptr(ses.h), d, w.dtype, s))
+            else:
+                check(L.mtj_gemm_splitk(ptr(ses.act), d + F, ptr(w.w_out[i]), ptr(w.b2[i]), B, d, d + F, w.dtype,
+                                        EPI_RESID, ptr(ses.x), d, F32, ptr(ses.gemm_work), ses.gemm_work.numel(), s))
 
     def sample_greedy(self, ses, out_tokens, embed_next=True):
         check(_abi.lib().mtj_sample_greedy(ptr(ses.logits), ses.B, self.w.V, ptr(ses.tok), ptr(out_tokens),

@@ -186,6 +186,37 @@ def test_gemm_splitk_matches_reference_and_is_deterministic(L, dt, M, N, K):
                                       a.ptr(work), nb - 4, S()))
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(32, 4096, 20480), (5, 512, 2560), (3, 64, 64), (8, 1024, 4096)])
+def test_gemm_splitk_with_the_following_layernorm(L, dt, M, N, K):
+    """The residual reduce that also normalises the rows it completes: x as from mtj_gemm_splitk (bit for bit), h as
+    ReplicatedLayerNorm of that x."""
+    a = abi()
+    g = torch.Generator().manual_seed(M * 7 + N + K)
+    A = torch.randn(M, K, generator=g).to(TD[dt]).to(DEV)
+    Wh = (torch.randn(K, N, generator=g) * 0.05).to(TD[dt]).to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    sc = (1 + 0.1 * torch.randn(N, generator=g)).to(DEV)
+    of = (0.1 * torch.randn(N, generator=g)).to(DEV)
+    W = _packed(Wh)
+    code = a.dtype_code(TD[dt])
+    nb = L.mtj_gemm_splitk_work_bytes(M, N, K, code)
+    work = torch.empty(max(nb, 16), dtype=torch.uint8, device=DEV)
+    x0 = torch.randn(M, N, generator=g).to(DEV)
+    x_ref = x0.clone()
+    a.check(L.mtj_gemm_splitk(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_RESID, a.ptr(x_ref), N, 0,
+                              a.ptr(work), work.numel(), S()))
+    for h_dt in ("f32", "bf16"):
+        x = x0.clone()
+        h = torch.zeros(M, N, dtype=TD[h_dt], device=DEV)
+        a.check(L.mtj_gemm_splitk_ln(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.ptr(x), N, a.ptr(work),
+                                     work.numel(), a.ptr(sc), a.ptr(of), a.ptr(h), N, a.dtype_code(TD[h_dt]), S()))
+        torch.cuda.synchronize()
+        assert torch.equal(x, x_ref)
+        ref = O.replicated_layer_norm(x.double().cpu(), sc.double().cpu(), of.double().cpu()).to(DEV)
+        assert rel_err(h, ref) < (6e-6 if h_dt == "f32" else 4e-3)
+
+
 def test_gemm_rejects_bad_arguments(L):
     a = abi()
     A = torch.zeros(4, 48, device=DEV)

@@ -220,11 +220,17 @@ __global__ __launch_bounds__(SNT) void nucleus_kernel(const float* __restrict__ 
     if (t < nt) {
       const int j = jw + t * 64;
       const bool live = j < V;
-      const double e = live ? exp((double)val[t] - l0) / Z : 0.0;
-      const double incl = wave_inclusive(e);
-      const double before = base + (incl - e);
-      if (live && j > 0 && before > tp) removed |= 1ull << t;
-      base += __shfl(incl, 63);
+      if (base > tp) {
+        // the mass before this tile already exceeds top_p (base is the same in every lane, and it only grows):
+        // every rank of the tile is outside the nucleus, no exponential needed
+        if (live && j > 0) removed |= 1ull << t;
+      } else {
+        const double e = live ? exp((double)val[t] - l0) / Z : 0.0;
+        const double incl = wave_inclusive(e);
+        const double before = base + (incl - e);
+        if (live && j > 0 && before > tp) removed |= 1ull << t;
+        base += __shfl(incl, 63);
+      }
       if (live) {
         const uint32_t id = id_of(t);
         // the sort key folds -0.0 into +0.0: fetch the original bits for a zero
@@ -238,10 +244,16 @@ __global__ __launch_bounds__(SNT) void nucleus_kernel(const float* __restrict__ 
   }
   tmax = block_max(tmax, sh);
   // ---- inverse-CDF draw over exp(filtered / temp - max) in sorted order
+  // exp(x) is exactly 0 in float64 below -745.14: what the filter pushed down by 1e10 (almost every rank of a peaked
+  // distribution) needs no exponential
+  auto weight = [&](int t) {
+    const double x = (double)filtered_of(t, id_of(t), val[t]) / tmp - tmax;
+    return x < -746.0 ? 0.0 : exp(x);
+  };
   double wloc = 0.0;
 #pragma unroll
   for (int t = 0; t < NT_MAX; ++t)
-    if (t < nt && jw + t * 64 < V) wloc += exp((double)filtered_of(t, id_of(t), val[t]) / tmp - tmax);
+    if (t < nt && jw + t * 64 < V) wloc += weight(t);
   const double total = block_sum(wloc, sh);
   double cum = 0.0;
   for (int w = 0; w < wave; ++w) cum += sh[w];
@@ -251,7 +263,7 @@ __global__ __launch_bounds__(SNT) void nucleus_kernel(const float* __restrict__ 
   for (int t = 0; t < NT_MAX; ++t) {
     if (t < nt) {
       const int j = jw + t * 64;
-      const double w = (j < V) ? exp((double)filtered_of(t, id_of(t), val[t]) / tmp - tmax) : 0.0;
+      const double w = (j < V) ? weight(t) : 0.0;
       const double incl = wave_inclusive(w);
       if (w > 0.0) lastpos = j;
       if (cum + incl > target && j < V && first == 0x7fffffff) first = j;

@@ -440,6 +440,18 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
   const int nvalid = (pos[b] + 1 < Tcap) ? pos[b] + 1 : Tcap;
   const int ns = (nvalid + DEC_CHUNK - 1) / DEC_CHUNK;    // non-empty splits (<= S <= 64)
   const float* wb = work + bh * S * (DH + 2);
+  // The partial vectors do not depend on the weights: thread e requests element e of the first 16 partials before
+  // the barrier behind which the weights are visible, so the merge costs one memory round trip after the weights'
+  // own, not one per four splits.  (d_head <= 256: one element per thread.)
+  static_assert(DH <= 256, "one element per thread");
+  constexpr int G = 16;
+  const int e = tid;
+  float pv[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const int s2 = g < ns ? g : ns - 1;                      // beyond the last split: a valid address, weight 0 below
+    pv[g] = (e < DH) ? wb[(int64_t)s2 * (DH + 2) + 2 + e] : 0.f;
+  }
   if (tid < 64) {
     const float ms = (tid < ns) ? wb[(int64_t)tid * (DH + 2)] : -INFINITY;
     const float ls = (tid < ns) ? wb[(int64_t)tid * (DH + 2) + 1] : 0.f;
@@ -449,16 +461,24 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
     wgt[tid] = f / lt;
   }
   __syncthreads();
-  for (int e = tid; e < DH; e += 256) {
+  if (e < DH) {
     float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    int s2 = 0;
-    for (; s2 + 3 < ns; s2 += 4) {
-      a0 += wgt[s2] * wb[(int64_t)s2 * (DH + 2) + 2 + e];
-      a1 += wgt[s2 + 1] * wb[(int64_t)(s2 + 1) * (DH + 2) + 2 + e];
-      a2 += wgt[s2 + 2] * wb[(int64_t)(s2 + 2) * (DH + 2) + 2 + e];
-      a3 += wgt[s2 + 3] * wb[(int64_t)(s2 + 3) * (DH + 2) + 2 + e];
+    for (int s0 = 0; s0 < ns; s0 += G) {
+      if (s0 > 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const int s2 = s0 + g < ns ? s0 + g : ns - 1;
+          pv[g] = wb[(int64_t)s2 * (DH + 2) + 2 + e];
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < G; g += 4) {
+        a0 += (s0 + g < ns ? wgt[s0 + g] : 0.f) * pv[g];
+        a1 += (s0 + g + 1 < ns ? wgt[s0 + g + 1] : 0.f) * pv[g + 1];
+        a2 += (s0 + g + 2 < ns ? wgt[s0 + g + 2] : 0.f) * pv[g + 2];
+        a3 += (s0 + g + 3 < ns ? wgt[s0 + g + 3] : 0.f) * pv[g + 3];
+      }
     }
-    for (; s2 < ns; ++s2) a0 += wgt[s2] * wb[(int64_t)s2 * (DH + 2) + 2 + e];
     store_as(out, (int64_t)b * ld_out + h * DH + e, (a0 + a1) + (a2 + a3), out_dtype);
   }
 }

@@ -72,9 +72,13 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   const bool pairs = a.epi == MTJ_EPI_INPROJ;
   const int64_t upw = pairs ? 2 : 1;
   const int64_t units = a.N / upw;
-  const int64_t gw = (int64_t)blockIdx.x * nwaves + wave, nw_total = (int64_t)gridDim.x * nwaves;
-  const int64_t row0 = (units * gw / nw_total) * upw, row1 = (units * (gw + 1) / nw_total) * upw;
-  const int nrows = (int)(row1 - row0);                     // <= 64 (the host sizes the grid for that)
+  // The units of a workgroup (an equal contiguous share of all) go to its wavefronts in contiguous runs, the odd
+  // ones to the FIRST wavefronts: under a saturated memory system the wavefronts of a SIMD are served oldest
+  // first and the youngest finish last, so they should be the ones with less to do.
+  const int64_t ub0 = units * blockIdx.x / gridDim.x, ub1 = units * (blockIdx.x + 1) / gridDim.x;
+  const int cnt = (int)(ub1 - ub0), per = cnt / nwaves, rem = cnt % nwaves;
+  const int64_t row0 = (ub0 + (int64_t)wave * per + (wave < rem ? wave : rem)) * upw;
+  const int nrows = (per + (wave < rem ? 1 : 0)) * (int)upw;   // <= 64 (the host sizes the grid for that)
 
   // ---- x first (4 values per thread while K <= 4096; the general loop below covers the rest) ...
   const bool ln = a.ln_scale != nullptr;

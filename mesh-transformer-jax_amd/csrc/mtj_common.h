@@ -4,6 +4,8 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <atomic>
+#include <mutex>
 #include "mtj_abi.h"
 
 typedef __bf16 bf16_t;
@@ -26,6 +28,40 @@ int mtj_check_launch(const char* what);
   } while (0)
 
 static inline bool mtj_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Set-up that has to run once per device and process (kernel attributes, symbol addresses): f(device) runs under a
+// lock the first time the calling thread's current device reaches this point; later calls cost one hipGetDevice
+// and one atomic load.  Thread-safe; a failed f is retried by the next call.
+constexpr int MTJ_MAX_DEVICES = 64;
+struct mtj_device_once {
+  std::atomic<uint64_t> done{0};
+  std::mutex mu;
+};
+template <class F>
+static inline int mtj_once_per_device(mtj_device_once& o, const char* who, F&& f) {
+  int dev = 0;
+  const hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+  if (dev < 0 || dev >= MTJ_MAX_DEVICES) return mtj_fail(MTJ_ELIMIT, "%s: device index %d is beyond %d", who, dev, MTJ_MAX_DEVICES);
+  const uint64_t bit = 1ull << dev;
+  if (o.done.load(std::memory_order_acquire) & bit) return MTJ_OK;
+  std::lock_guard<std::mutex> guard(o.mu);
+  if (o.done.load(std::memory_order_relaxed) & bit) return MTJ_OK;
+  const int rc = f(dev);
+  if (rc == MTJ_OK) o.done.fetch_or(bit, std::memory_order_release);
+  return rc;
+}
+
+// Raises the dynamic-LDS limit of `kernel` once per device.
+template <class K>
+static inline int mtj_allow_lds(mtj_device_once& o, const char* who, K kernel, size_t bytes) {
+  return mtj_once_per_device(o, who, [&](int) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "%s: hipFuncSetAttribute: %s", who, hipGetErrorString(e));
+    return (int)MTJ_OK;
+  });
+}
 
 // ---------------------------------------------------------------- device helpers
 // bf16 <-> f32.  Rounding to bf16 is round-to-nearest-even (what jnp.astype(bfloat16) does).

@@ -536,13 +536,8 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
 template <int EPI>
 int launch_dma(const gemm_args& a, hipStream_t s) {
   constexpr size_t lds = 2 * 2 * 256 * 64 * 2;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_dma_kernel<EPI>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_gemm: hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_set = true;
-  }
+  static mtj_device_once once;
+  if (int rc = mtj_allow_lds(once, "mtj_gemm", &gemm_dma_kernel<EPI>, lds)) return rc;
   const int tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
   gemm_dma_kernel<EPI><<<dim3(tiles, a.splits), 512, lds, s>>>(a);
   return mtj_check_launch("mtj_gemm");
@@ -554,13 +549,8 @@ int launch(const gemm_args& a, hipStream_t s) {
   constexpr size_t lds = 2 * (size_t)(BM + BN) * (BK + mma<T>::EPC) * sizeof(T);
   static_assert(lds <= 160 * 1024, "tile does not fit LDS");
   static_assert(lds >= 2 * BM * sizeof(int) + WAVES_M * WAVES_N * 32 * 36 * sizeof(float), "epilogue scratch does not fit");
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK, NS>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_gemm: hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_set = true;
-  }
+  static mtj_device_once once;
+  if (int rc = mtj_allow_lds(once, "mtj_gemm", &gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK, NS>, lds)) return rc;
   const int tiles = ((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   gemm_kernel<T, EPI, WAVES_M, WAVES_N, WM, WN, BK, NS><<<dim3(tiles, a.splits), WAVES_M * WAVES_N * 64, lds, s>>>(a);
   return mtj_check_launch("mtj_gemm");

@@ -243,13 +243,8 @@ int launch(const gemv_args& a, hipStream_t s) {
   if (grid < 1) grid = 1;
   const int64_t upw = a.epi == MTJ_EPI_INPROJ ? 2 : 1;
   while ((units + grid * 16 - 1) / (grid * 16) * upw > 62) grid *= 2;   // a lane per row: <= 64 rows per wavefront
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<T, U, FULL>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256);
-    if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_gemv: hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_set = true;
-  }
+  static mtj_device_once once;
+  if (int rc = mtj_allow_lds(once, "mtj_gemv", &gemv_kernel<T, U, FULL>, 160 * 1024 - 256)) return rc;
   gemv_kernel<T, U, FULL><<<(unsigned)grid, 1024, lds, s>>>(a);
   return mtj_check_launch("mtj_gemv");
 }

@@ -155,6 +155,18 @@ int mtj_attn_decode(const float* q, const void* k_cache, const void* v_cache, co
                     int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
                     void* work, void* stream);
 
+/* mtj_attn_decode for callers that cannot allocate or carry a workspace (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The partial results
+ * live in a device array built into the library (MTJ_ATTN_DECODE_STATIC_BYTES per device, held until the process
+ * ends); the call allocates nothing and returns MTJ_ELIMIT when mtj_attn_decode_work_bytes(B, H, dh, Tcap) exceeds
+ * that.  Same arguments and results as mtj_attn_decode otherwise.  Every call on a device shares the array: calls
+ * that overlap on one device (two streams, two threads) race. */
+#define MTJ_ATTN_DECODE_STATIC_BYTES (20 * 1024 * 1024)
+int64_t mtj_attn_decode_static_max_bytes(void);
+int mtj_attn_decode_static(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,
+                           int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
+                           void* stream);
+
 /* Next-step embedding fused into the samplers: when `w` is non-NULL the sampler also writes
  * x_next[b, :] = w[token, :] + bias (EmbeddingShard of the token it just chose, layers.py:187-202), which is the
  * input of the next decode step (transformer_shard.py:107). */

@@ -504,13 +504,8 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
   do {                                                                                                               \
     constexpr size_t lds = 2 * ((size_t)BKV * (DH + mma<T>::EPC) + (size_t)DH * (BKV + mma<T>::EPC)) * sizeof(T);    \
     static_assert(lds <= 160 * 1024, "attention tiles do not fit LDS");                                              \
-    static bool attr_set = false;                                                                                    \
-    if (!attr_set) {                                                                                                 \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<T, DH, NW, BKV>),        \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                      \
-      if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_attn_prefill: hipFuncSetAttribute: %s", hipGetErrorString(e)); \
-      attr_set = true;                                                                                               \
-    }                                                                                                                \
+    static mtj_device_once once;                                                                                     \
+    if (int rc = mtj_allow_lds(once, "mtj_attn_prefill", &attn_prefill_kernel<T, DH, NW, BKV>, lds)) return rc;      \
     const int64_t nqblk = (Tp + NW * 32 - 1) / (NW * 32);                                                            \
     MTJ_REQUIRE(nqblk * H * B < (1ll << 31), MTJ_ELIMIT, "mtj_attn_prefill: too many workgroups");                    \
     attn_prefill_kernel<T, DH, NW, BKV><<<(unsigned)(nqblk * H * B), NW * 64, lds, s>>>(                              \
@@ -530,17 +525,18 @@ extern "C" int64_t mtj_attn_decode_work_bytes(int64_t B, int64_t H, int64_t dh, 
   return B * H * (int64_t)decode_splits(Tcap) * (dh + 2) * (int64_t)sizeof(float);
 }
 
-extern "C" int mtj_attn_decode(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,
-                               int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
-                               void* work, void* stream) {
-  MTJ_REQUIRE(q && k_cache && v_cache && pos && out && work, MTJ_EINVAL, "mtj_attn_decode: null pointer");
-  MTJ_REQUIRE(B > 0 && H > 0 && Tcap > 0 && ld_out >= H * dh && B < 65536 && H < 65536, MTJ_EINVAL,
-              "mtj_attn_decode: bad shape");
-  MTJ_REQUIRE(out_dtype == MTJ_F32 || out_dtype == MTJ_BF16, MTJ_EDTYPE, "mtj_attn_decode: out_dtype %d", out_dtype);
+namespace {
+
+int attn_decode_impl(const char* who, const float* q, const void* k_cache, const void* v_cache, const int32_t* pos,
+                     int64_t B, int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
+                     void* work, void* stream) {
+  MTJ_REQUIRE(q && k_cache && v_cache && pos && out && work, MTJ_EINVAL, "%s: null pointer", who);
+  MTJ_REQUIRE(B > 0 && H > 0 && Tcap > 0 && ld_out >= H * dh && B < 65536 && H < 65536, MTJ_EINVAL, "%s: bad shape", who);
+  MTJ_REQUIRE(out_dtype == MTJ_F32 || out_dtype == MTJ_BF16, MTJ_EDTYPE, "%s: out_dtype %d", who, out_dtype);
   MTJ_REQUIRE(mtj_aligned16(q) && mtj_aligned16(k_cache) && mtj_aligned16(v_cache) && mtj_aligned16(work), MTJ_EALIGN,
-              "mtj_attn_decode: pointers must be 16-byte aligned");
+              "%s: pointers must be 16-byte aligned", who);
   const int S = decode_splits(Tcap);
-  MTJ_REQUIRE(S <= 64, MTJ_ELIMIT, "mtj_attn_decode: window of %lld slots exceeds %d", (long long)Tcap, 64 * DEC_CHUNK);
+  MTJ_REQUIRE(S <= 64, MTJ_ELIMIT, "%s: window of %lld slots exceeds %d", who, (long long)Tcap, 64 * DEC_CHUNK);
   float* partials = reinterpret_cast<float*>(work);
   dim3 grid((unsigned)S, (unsigned)H, (unsigned)B);
   hipStream_t s = (hipStream_t)stream;
@@ -555,7 +551,65 @@ extern "C" int mtj_attn_decode(const float* q, const void* k_cache, const void* 
   else if (dtype == MTJ_BF16 && dh == 64) MTJ_DECODE(bf16_t, 64);
   else if (dtype == MTJ_F32 && dh == 256) MTJ_DECODE(float, 256);
   else if (dtype == MTJ_F32 && dh == 64) MTJ_DECODE(float, 64);
-  else return mtj_fail(MTJ_EINVAL, "mtj_attn_decode: unsupported dtype %d / d_head %lld (64 or 256)", dtype, (long long)dh);
+  else return mtj_fail(MTJ_EINVAL, "%s: unsupported dtype %d / d_head %lld (64 or 256)", who, dtype, (long long)dh);
 #undef MTJ_DECODE
-  return mtj_check_launch("mtj_attn_decode");
+  return mtj_check_launch(who);
+}
+
+}  // namespace
+
+extern "C" int mtj_attn_decode(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,
+                               int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
+                               void* work, void* stream) {
+  return attn_decode_impl("mtj_attn_decode", q, k_cache, v_cache, pos, B, H, Tcap, dh, out, ld_out, out_dtype, dtype, work,
+                          stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same two launches with the partial results kept in a device array that lives in the code object, for
+// callers that cannot allocate (or pass) a workspace.  Every device that loads the library holds its own copy of
+// `scratch` at its own address: the address is looked up once per device (hipGetSymbolAddress with that device
+// current) and that pointer, never the array's name, is what host code hands to the kernels.  Nothing in
+// `scratch` has to start at zero: the merge kernel reads only the partials that the first kernel of the same
+// call has written.  All calls on one device share the array, so calls that overlap on one device race.
+static __device__ __align__(256) unsigned char scratch[MTJ_ATTN_DECODE_STATIC_BYTES];
+
+namespace {
+mtj_device_once scratch_once;
+void* scratch_ptr[MTJ_MAX_DEVICES];
+
+int scratch_address(void** p) {
+  int dev = 0;
+  const int rc = mtj_once_per_device(scratch_once, "mtj_attn_decode_static", [&](int d) {
+    void* sym = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !sym)
+      return mtj_fail(MTJ_EHIP, "mtj_attn_decode_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    scratch_ptr[d] = sym;
+    return (int)MTJ_OK;
+  });
+  if (rc) return rc;
+  const hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_attn_decode_static: hipGetDevice: %s", hipGetErrorString(e));
+  *p = scratch_ptr[dev];
+  return MTJ_OK;
+}
+}  // namespace
+
+extern "C" int64_t mtj_attn_decode_static_max_bytes(void) { return MTJ_ATTN_DECODE_STATIC_BYTES; }
+
+extern "C" int mtj_attn_decode_static(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos,
+                                      int64_t B, int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out,
+                                      int out_dtype, int dtype, void* stream) {
+  MTJ_REQUIRE(B > 0 && H > 0 && Tcap > 0 && dh > 0, MTJ_EINVAL, "mtj_attn_decode_static: bad shape");
+  const int64_t need = mtj_attn_decode_work_bytes(B, H, dh, Tcap);
+  MTJ_REQUIRE(need <= MTJ_ATTN_DECODE_STATIC_BYTES, MTJ_ELIMIT,
+              "mtj_attn_decode_static: B=%lld H=%lld Tcap=%lld dh=%lld needs %lld bytes of partial results, the built-in "
+              "array holds %lld; use mtj_attn_decode with a caller-provided workspace",
+              (long long)B, (long long)H, (long long)Tcap, (long long)dh, (long long)need,
+              (long long)MTJ_ATTN_DECODE_STATIC_BYTES);
+  void* work = nullptr;
+  if (int rc = scratch_address(&work)) return rc;
+  return attn_decode_impl("mtj_attn_decode_static", q, k_cache, v_cache, pos, B, H, Tcap, dh, out, ld_out, out_dtype,
+                          dtype, work, stream);
 }

@@ -49,6 +49,8 @@ SIGNATURES = {
     "mtj_attn_prefill": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64, _i32, _p, _p]),
     "mtj_attn_decode_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "mtj_attn_decode": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _i32, _i32, _p, _p]),
+    "mtj_attn_decode_static_max_bytes": (_i64, []),
+    "mtj_attn_decode_static": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _i32, _i32, _p]),
     "mtj_sample_greedy": (_i32, [_p, _i64, _i64, _p, _p, _i64, _p, _p, C.POINTER(NextEmbed), _p]),
     "mtj_sample_work_bytes": (_i64, [_i64, _i64]),
     "mtj_sample_nucleus": (_i32, [_p, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p,

@@ -92,7 +92,7 @@ def time_dominant_kernel(net, ses, reps=20):
         for i in w.layer_ids:
             ip = eng._inproj(ses, i, 1, ses.pos, ses.q, F32, ses.act, F32, None)
             check(L.mtj_gemv(ptr(ses.x), ptr(w.ln_s[i]), ptr(w.ln_o[i]), ptr(w.w_in[i]), ptr(w.b1[i]), 3 * d + F, d,
-                             w.dtype, EPI_INPROJ, None, 0, C.byref(ip), s))
+                             w.dtype, EPI_INPROJ, None, 0, C.byref(ip), None, s))
 
     sweep()
     torch.cuda.synchronize()
@@ -193,7 +193,7 @@ def pmc_probe(dev):
         for i in w.layer_ids:
             ip = eng._inproj(ses, i, 1, ses.pos, ses.q, F32, ses.act, F32, None)
             check(L.mtj_gemv(ptr(ses.x), ptr(w.ln_s[i]), ptr(w.ln_o[i]), ptr(w.w_in[i]), ptr(w.b1[i]), 3 * w.d + w.F, w.d,
-                             w.dtype, EPI_INPROJ, None, 0, C.byref(ip), s))
+                             w.dtype, EPI_INPROJ, None, 0, C.byref(ip), None, s))
     torch.cuda.synchronize()
     print("pmc probe done")
 

@@ -13,7 +13,12 @@
  *   - return value: 0 on success, a negative MTJ_E* code otherwise; mtj_last_error() returns the
  *     message of the calling thread's last failure;
  *   - activations are float32 unless `dtype` says otherwise; `dtype` selects the storage type of
- *     weights / K,V cache / GEMM inputs: MTJ_F32 (exact path) or MTJ_BF16;
+ *     weights / K,V cache / GEMM inputs: MTJ_F32 (exact path), MTJ_BF16 or MTJ_F16.  The reference multiplies
+ *     float32 activations with bf16 weights (jnp.dot(f32, bf16)); the matrix cores want both operands in one
+ *     16-bit type, and float16 holds every bf16 weight exactly (after a power-of-two scale, see
+ *     mtj_pack_weight_cvt) while rounding an activation to 11 significant bits instead of bf16's 8, so the
+ *     matrix-core paths of a bf16 model run in MTJ_F16;
+ *   - conversions to MTJ_F16 saturate at +-65504;
  *   - "packed" weights are row-major [N_out, K_in] (K contiguous), i.e. the transpose of haiku's
  *     [in, out]; mtj_pack_weight builds them, with row/column offsets so that q|v|k|fc_in are
  *     concatenated along N and out|fc_out along K.
@@ -27,9 +32,9 @@
 extern "C" {
 #endif
 
-#define MTJ_ABI_VERSION 1
+#define MTJ_ABI_VERSION 2
 
-enum { MTJ_F32 = 0, MTJ_BF16 = 1 };
+enum { MTJ_F32 = 0, MTJ_BF16 = 1, MTJ_F16 = 2 };
 
 enum {
   MTJ_OK = 0,
@@ -66,14 +71,25 @@ typedef struct {
   const float* cos_tab;                 /* [max_pos, r/2]                                              */
   void* q;                              /* [B, H, Tp, dh] in q_dtype                                   */
   int32_t q_dtype;                      /* MTJ_F32 (decode attention reads float32 q) or MTJ_BF16      */
-  void* k_cache;                        /* [B, H, Tcap, dh] dtype, rotated keys                        */
-  void* v_cache;                        /* [B, H, Tcap, dh] dtype                                      */
-  void* v_t;                            /* optional [B, H, dh, ldvt] dtype: V transposed, for prefill  */
+  int32_t kv_dtype;                     /* storage type of k_cache, v_cache and v_t                    */
+  void* k_cache;                        /* [B, H, Tcap, dh] kv_dtype, rotated keys                     */
+  void* v_cache;                        /* [B, H, Tcap, dh] kv_dtype                                   */
+  void* v_t;                            /* optional [B, H, dh, ldvt] kv_dtype: V transposed, for prefill */
   int64_t ldvt;                         /* row length of v_t: >= Tp rounded up to a multiple of 64     */
   void* act;                            /* [M, ld_act]: gelu(fc_in) goes to columns [d, d+F)           */
   int64_t ld_act;
   int32_t act_dtype;                    /* MTJ_F32 or MTJ_BF16                                         */
 } mtj_inproj;
+
+/*
+ * Per-range partial results of one-token attention, as mtj_attn_decode_partials leaves them and mtj_gemv consumes them:
+ * partials[((b*H + h)*splits + s) * (dh + 4)] = {max, sum, -, -, V[dh]}; the attention output of a (sequence, head) is
+ * sum_s exp(max_s - max) V_s / sum_s exp(max_s - max) sum_s.
+ */
+typedef struct {
+  const float* partials;
+  int32_t n_heads, d_head, splits;
+} mtj_attn_merge;
 
 /*
  * Transpose-pack a haiku [K, N] weight (row stride src_ld) into dst[(n_off + n) * K_total + k_off + k].
@@ -82,6 +98,14 @@ typedef struct {
  */
 int mtj_pack_weight(const void* src, int64_t src_ld, int64_t K, int64_t N, void* dst, int64_t K_total,
                     int64_t n_off, int64_t k_off, int dtype, void* stream);
+
+/* mtj_pack_weight with a change of type: dst (dst_dtype) = src (src_dtype) * scale, rounded to nearest even
+ * (saturating for MTJ_F16).  With src bf16, dst float16 and `scale` a power of two that brings the largest weight
+ * of the matrix below 65504, every weight whose scaled magnitude is at least 2^-14 is represented exactly; smaller
+ * ones are rounded to a multiple of 2^-24 (below 2^-40 of the largest weight).  The matching mtj_gemm call passes
+ * alpha = 1 / scale. */
+int mtj_pack_weight_cvt(const void* src, int64_t src_ld, int64_t K, int64_t N, void* dst, int64_t K_total,
+                        int64_t n_off, int64_t k_off, int src_dtype, int dst_dtype, float scale, void* stream);
 
 /* out[m, :] = W[tok[m], :] + b  (EmbeddingShard.__call__, layers.py:187-202: one_hot @ W + b).
  * W is the tree leaf itself, [V, d] in `dtype`; b float32 [d]; out float32 [M, d].
@@ -101,11 +125,13 @@ int mtj_layernorm(const float* x, const float* scale, const float* offset, int64
 int mtj_xent(const float* logits, int64_t ld, const int32_t* target, int64_t M, int64_t V, float* loss,
              uint8_t* correct, void* stream);
 
-/* C = A[M, K] (dtype, row stride lda) x W[N, K]^T (packed, dtype) with epilogue `epi`.
- * hk.Linear call sites: layers.py:249-258, 559.  MFMA kernel; bias is float32 [N] or NULL.
+/* C = alpha * A[M, K] (dtype, row stride lda) x W[N, K]^T (packed, dtype) with epilogue `epi`.
+ * hk.Linear call sites: layers.py:249-258, 559.  MFMA kernel; bias is float32 [N] or NULL; alpha undoes the scale
+ * of mtj_pack_weight_cvt (1 otherwise) and multiplies the float32 accumulator before anything else is applied.
  * STORE: out [M, ldo] in out_dtype.  RESID: out float32 [M, ldo].  INPROJ: `ip` non-NULL, bias = b1 [F]. */
 int mtj_gemm(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
-             int dtype, int epi, void* out, int64_t ldo, int out_dtype, const mtj_inproj* ip, void* stream);
+             int dtype, int epi, void* out, int64_t ldo, int out_dtype, const mtj_inproj* ip, float alpha,
+             void* stream);
 
 /* mtj_gemm for problems with few output tiles (batched decode; the out projection of a short prompt): when the
  * output has too few tiles to occupy the
@@ -117,7 +143,7 @@ int mtj_gemm(const void* A, int64_t lda, const void* W, const float* bias, int64
 int64_t mtj_gemm_splitk_work_bytes(int64_t M, int64_t N, int64_t K, int dtype);
 int mtj_gemm_splitk(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
                     int dtype, int epi, void* out, int64_t ldo, int out_dtype, void* work, int64_t work_bytes,
-                    void* stream);
+                    float alpha, void* stream);
 
 /* mtj_gemm_splitk with the RESID epilogue, followed in the same launch by the LayerNorm of the rows it completes:
  * x [M, ldx] float32 += A x W^T + bias, then h [M, ldh] (h_dtype) = ReplicatedLayerNorm(x) with ln_scale / ln_offset
@@ -125,15 +151,17 @@ int mtj_gemm_splitk(const void* A, int64_t lda, const void* W, const float* bias
  * generate_once (transformer_shard.py:97-115).  `work` as for mtj_gemm_splitk; N <= 16384. */
 int mtj_gemm_splitk_ln(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
                        int dtype, float* x, int64_t ldx, void* work, int64_t work_bytes, const float* ln_scale,
-                       const float* ln_offset, void* h, int64_t ldh, int h_dtype, void* stream);
+                       const float* ln_offset, void* h, int64_t ldh, int h_dtype, float alpha, void* stream);
 
 /* Batch-1 decode matrix-vector product: y = f(x) @ W^T with float32 activations and float32 accumulation
  * (jnp.dot(f32, bf16) semantics of hk.Linear at decode, layers.py:316-344).  x float32 [K].
  * If ln_scale != NULL the kernel first applies LayerNorm(x) (layers.py:17-36) - x then has K = d entries.
+ * If am != NULL (no LayerNorm then) the first am->n_heads * am->d_head entries of the input are not read from x but
+ * merged from the attention partials of batch row 0 (mtj_attn_decode_partials).
  * Same epilogues as mtj_gemm with M = 1. */
 int mtj_gemv(const float* x, const float* ln_scale, const float* ln_offset, const void* W, const float* bias,
              int64_t N, int64_t K, int dtype, int epi, void* out, int out_dtype, const mtj_inproj* ip,
-             void* stream);
+             const mtj_attn_merge* am, void* stream);
 
 /* Causal self-attention over a left-padded rectangle (self_attn + masks of get_init_decode_state,
  * layers.py:260-285, 347-366).  q [B,H,Tp,dh], k_cache [B,H,Tcap,dh] (rotated), v_t [B,H,dh,ldvt] with
@@ -148,20 +176,30 @@ int mtj_attn_prefill(const void* q, const void* k_cache, const void* v_t, const 
 
 /* One-token attention over the K/V window (decode_once, layers.py:316-344): for sequence b the valid
  * slots are [0, min(pos[b]+1, Tcap)).  q float32 [B,H,dh]; caches in `dtype`; out [B, ld_out] in out_dtype
- * (columns h*dh + c).  `work` (16-byte aligned, mtj_attn_decode_work_bytes(B, H, dh, Tcap) bytes) holds the per-split
- * partial results between the two launches this call makes; calls sharing one `work` must not overlap. */
+ * (columns h*dh + c).  The valid slots of a (sequence, head) are cut into mtj_attn_decode_splits(B, H, Tcap) equal key
+ * ranges that run as separate workgroups; `work` (16-byte aligned, mtj_attn_decode_work_bytes(B, H, dh, Tcap) bytes)
+ * holds their partial results (max, sum, weighted V) until a second launch merges them (no second launch when there
+ * is one range); calls sharing one `work` must not overlap. */
+int mtj_attn_decode_splits(int64_t B, int64_t H, int64_t Tcap);
 int64_t mtj_attn_decode_work_bytes(int64_t B, int64_t H, int64_t dh, int64_t Tcap);
 int mtj_attn_decode(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,
                     int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
                     void* work, void* stream);
 
+/* The partial results of mtj_attn_decode without the merge: mtj_gemv merges them while it stages its input (the
+ * attention output is consumed by the out projection only, layers.py:285), which saves a launch and a round trip
+ * through memory per layer at batch 1.  *merge is filled for mtj_gemv. */
+int mtj_attn_decode_partials(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,
+                             int64_t H, int64_t Tcap, int64_t dh, int dtype, void* work, mtj_attn_merge* merge,
+                             void* stream);
+
 /* mtj_attn_decode for callers that cannot allocate or carry a workspace (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The partial results
  * live in a device array built into the library (MTJ_ATTN_DECODE_STATIC_BYTES per device, held until the process
- * ends); the call allocates nothing and returns MTJ_ELIMIT when mtj_attn_decode_work_bytes(B, H, dh, Tcap) exceeds
+ * ends: room for 4032 (sequence, head) pairs at d_head 256, e.g. batch 252 of a 16-head model); the call allocates nothing and returns MTJ_ELIMIT when mtj_attn_decode_work_bytes(B, H, dh, Tcap) exceeds
  * that.  Same arguments and results as mtj_attn_decode otherwise.  Every call on a device shares the array: calls
  * that overlap on one device (two streams, two threads) race. */
-#define MTJ_ATTN_DECODE_STATIC_BYTES (20 * 1024 * 1024)
+#define MTJ_ATTN_DECODE_STATIC_BYTES (4 * 1024 * 1024)
 int64_t mtj_attn_decode_static_max_bytes(void);
 int mtj_attn_decode_static(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,
                            int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,

@@ -28,6 +28,30 @@ template <> struct mma<bf16_t> {
     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
   }
 };
+template <> struct mma<f16_t> {
+  static constexpr int EPC = 8;
+  typedef uint16_t raw_t;
+  struct frag { f16x8 v; };
+  __device__ static __forceinline__ frag load(const f16_t* p) {
+    frag f;
+    f.v = *reinterpret_cast<const f16x8*>(p);
+    return f;
+  }
+  __device__ static __forceinline__ void pin(frag& f) { asm volatile("" : "+v"(f.v)); }
+  __device__ static __forceinline__ frag from_floats(const float* p) {
+    frag f;
+    uint32x4 u;
+    u.x = pack_f16x2(p[0], p[1]);
+    u.y = pack_f16x2(p[2], p[3]);
+    u.z = pack_f16x2(p[4], p[5]);
+    u.w = pack_f16x2(p[6], p[7]);
+    f.v = *reinterpret_cast<f16x8*>(&u);
+    return f;
+  }
+  __device__ static __forceinline__ void run(floatx16& c, const frag& a, const frag& b) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.v, b.v, c, 0, 0, 0);
+  }
+};
 template <> struct mma<float> {
   static constexpr int EPC = 4;
   typedef uint32_t raw_t;
@@ -309,10 +333,10 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
 #pragma unroll
       for (int v4 = 0; v4 < 4; ++v4) {
         const int e = i * 32 + 8 * v4 + 4 * fg;
-        if (sizeof(T) == 2) {
+        if constexpr (sizeof(T) == 2) {
           uint32x2 pk;
-          pk.x = pack_bf16x2(o[i][v4 * 4] * inv, o[i][v4 * 4 + 1] * inv);
-          pk.y = pack_bf16x2(o[i][v4 * 4 + 2] * inv, o[i][v4 * 4 + 3] * inv);
+          pk.x = pack2<T>(o[i][v4 * 4] * inv, o[i][v4 * 4 + 1] * inv);
+          pk.y = pack2<T>(o[i][v4 * 4 + 2] * inv, o[i][v4 * 4 + 3] * inv);
           *reinterpret_cast<uint32x2*>(op + e) = pk;
         } else {
           *reinterpret_cast<floatx4*>(op + e) =
@@ -323,167 +347,185 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
 }
 
 // ------------------------------------------------------------------------------------------------
-// Decode.  Grid (splits, H, B); each workgroup reduces 64 window slots to a partial (max, sum, weighted V)
-// and attn_combine_kernel merges the non-empty partials of a (sequence, head).  (Merging in the same launch,
-// by the last workgroup to arrive, needs a device-scope fence per workgroup; on this multi-die GPU that
-// fence writes back the L2 and made the kernel 6x slower than the two launches.)  16-byte loads: LPK lanes
-// cover one key row; all K and V loads of a workgroup are requested up front (V does not depend on the
-// scores).
-constexpr int DEC_CHUNK = 64;
+// Decode.  Grid (S, H, B): the valid part of a (sequence, head) window is cut into S equal key ranges (the cut
+// follows the position read from device memory, so every workgroup has work whatever the fill), and each
+// 4-wavefront workgroup reduces its range to a partial (max, sum, weighted V).  A wavefront owns every fourth
+// group of KPL keys and keeps its own online-softmax state in registers: LPK lanes cover one key row with 16-byte
+// loads, the score of a key is reduced over those lanes by shuffles, and the probability-weighted V rows are
+// accumulated per lane, so nothing crosses wavefronts until the end of the range.  All K and V rows of one
+// 64-key step are requested before the first is used and the next step's rows before the current step is
+// reduced; rows beyond the range are clamped to its last key and masked, so no load is conditional.
+//
+// Partials: work[((b*H + h)*S + s) * (DH + 4)] = {max, sum, -, -, V[DH]}.  With S == 1 and `out` given the normalised
+// result goes straight to `out`; otherwise attn_combine_kernel (or the prologue of the out-projection GEMV) merges them.
+constexpr int DEC_NI = 8;            // K (and V) loads per lane and step
+constexpr int DEC_PAD = MTJ_DEC_PAD;  // floats in front of the vector of a partial
+
+template <typename T> struct kvrow;   // one 16-byte piece of a cached row -> EPC floats
+template <> struct kvrow<float> {
+  static constexpr int EPC = 4;
+  __device__ static __forceinline__ void get(const uint32x4& w, float* f) {
+    f[0] = __uint_as_float(w.x); f[1] = __uint_as_float(w.y); f[2] = __uint_as_float(w.z); f[3] = __uint_as_float(w.w);
+  }
+};
+template <> struct kvrow<bf16_t> {
+  static constexpr int EPC = 8;
+  __device__ static __forceinline__ void get(const uint32x4& w, float* f) {
+    f[0] = bf16_lo(w.x); f[1] = bf16_hi(w.x); f[2] = bf16_lo(w.y); f[3] = bf16_hi(w.y);
+    f[4] = bf16_lo(w.z); f[5] = bf16_hi(w.z); f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
+  }
+};
+template <> struct kvrow<f16_t> {
+  static constexpr int EPC = 8;
+  __device__ static __forceinline__ void get(const uint32x4& w, float* f) {
+    f[0] = f16_lo(w.x); f[1] = f16_hi(w.x); f[2] = f16_lo(w.y); f[3] = f16_hi(w.y);
+    f[4] = f16_lo(w.z); f[5] = f16_hi(w.z); f[6] = f16_lo(w.w); f[7] = f16_hi(w.w);
+  }
+};
 
 template <typename T, int DH>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const T* __restrict__ kc,
                                                           const T* __restrict__ vc, const int32_t* __restrict__ pos,
-                                                          int H, int Tcap, float* __restrict__ work) {
-  constexpr int EPC = 16 / sizeof(T);
+                                                          int H, int Tcap, float* __restrict__ work, void* __restrict__ out,
+                                                          int64_t ld_out, int out_dtype) {
+  constexpr int EPC = kvrow<T>::EPC;
   constexpr int LPK = DH / EPC;      // lanes per key row
   constexpr int KPL = 64 / LPK;      // keys per wavefront load
-  constexpr int NI = DEC_CHUNK / (4 * KPL);   // loads per lane for K (and for V)
-  static_assert(LPK <= 64 && 64 % LPK == 0 && NI >= 1, "head dim does not map onto a wavefront");
-  __shared__ float sc[DEC_CHUNK];
+  constexpr int NI = DEC_NI;
+  constexpr int STEP = 4 * NI * KPL; // keys per workgroup step
+  static_assert(LPK <= 64 && 64 % LPK == 0, "head dim does not map onto a wavefront");
   __shared__ float part[4][DH];
+  __shared__ float stat[4][2];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z, S = gridDim.x;
   const int64_t bh = (int64_t)b * H + h;
-  const int nvalid = (pos[b] + 1 < Tcap) ? pos[b] + 1 : Tcap;
-  const int k0 = split * DEC_CHUNK;
-  const int nk = (k0 + DEC_CHUNK < nvalid) ? DEC_CHUNK : nvalid - k0;     // <= 0: nothing in this range
-  float* wout = work + (bh * S + split) * (DH + 2);
+  const int p = pos[b];
+  const int nvalid = (p + 1 < Tcap) ? p + 1 : Tcap;
+  const int per = (nvalid + S - 1) / S;                       // keys per range
+  const int k0 = split * per;
+  const int nk = (k0 + per <= nvalid) ? per : nvalid - k0;     // <= 0: an empty range (fewer keys than ranges)
   const int sub = lane / LPK, el = (lane % LPK) * EPC;
 
+  float m_run = -INFINITY, l_run = 0.f;                        // l_run and acc are per lane (their key subgroup)
+  float acc[EPC];
+#pragma unroll
+  for (int j = 0; j < EPC; ++j) acc[j] = 0.f;
+
   if (nk > 0) {
-    // ---- request every K and V row of the range
-    uint32x4 kr[NI], vr[NI];
     const T* kbase = kc + (bh * Tcap + k0) * DH + el;
     const T* vbase = vc + (bh * Tcap + k0) * DH + el;
+    uint32x4 kr[2][NI], vr[2][NI];
+    auto request = [&](int buf, int base) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int kk = (i * 4 + wave) * KPL + sub;
-      if (kk < nk) {
-        kr[i] = *reinterpret_cast<const uint32x4*>(kbase + (int64_t)kk * DH);
-        vr[i] = *reinterpret_cast<const uint32x4*>(vbase + (int64_t)kk * DH);
+      for (int i = 0; i < NI; ++i) {
+        int kk = base + (i * 4 + wave) * KPL + sub;
+        kk = kk < nk ? kk : nk - 1;
+        kr[buf][i] = *reinterpret_cast<const uint32x4*>(kbase + (int64_t)kk * DH);
+        vr[buf][i] = *reinterpret_cast<const uint32x4*>(vbase + (int64_t)kk * DH);
       }
-    }
+    };
     float qv[EPC];
+    request(0, 0);
 #pragma unroll
     for (int j = 0; j < EPC; ++j) qv[j] = q[bh * DH + el + j];
     const float scale = rsqrtf((float)DH);
-    // ---- scores
+    auto reduce = [&](int buf, int base) {
+      float sc[NI];
+      float mt = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int kk = (i * 4 + wave) * KPL + sub;
-      float d = 0.f;
-      if (kk < nk) {
-        const uint32x4 w = kr[i];
-        if (sizeof(T) == 2) {
-          d = bf16_lo(w.x) * qv[0] + bf16_hi(w.x) * qv[1 % EPC] + bf16_lo(w.y) * qv[2 % EPC] + bf16_hi(w.y) * qv[3 % EPC] +
-              bf16_lo(w.z) * qv[4 % EPC] + bf16_hi(w.z) * qv[5 % EPC] + bf16_lo(w.w) * qv[6 % EPC] + bf16_hi(w.w) * qv[7 % EPC];
-        } else {
-          d = __uint_as_float(w.x) * qv[0] + __uint_as_float(w.y) * qv[1] + __uint_as_float(w.z) * qv[2] +
-              __uint_as_float(w.w) * qv[3];
-        }
+      for (int i = 0; i < NI; ++i) {
+        float kf[EPC];
+        kvrow<T>::get(kr[buf][i], kf);
+        float d = 0.f;
+#pragma unroll
+        for (int j = 0; j < EPC; ++j) d = fmaf(kf[j], qv[j], d);
+#pragma unroll
+        for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o);
+        const int kk = base + (i * 4 + wave) * KPL + sub;
+        sc[i] = kk < nk ? d * scale : -INFINITY;
+        mt = fmaxf(mt, sc[i]);
       }
 #pragma unroll
-      for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o);
-      if (kk < nk && (lane % LPK) == 0) sc[kk] = d * scale;
-    }
-    __syncthreads();
-    // ---- softmax statistics of the range (64 scores: one wavefront's worth, every wavefront redoes it)
-    const float sv = (lane < nk) ? sc[lane] : -INFINITY;
-    const float m = wave_max(sv);
-    const float pv = (lane < nk) ? expf(sv - m) : 0.f;
-    const float l = wave_sum(pv);
-    // ---- weighted V from the registers
-    float acc[EPC];
+      for (int o = 32; o >= LPK; o >>= 1) mt = fmaxf(mt, __shfl_xor(mt, o));
+      const float m_new = fmaxf(m_run, mt);                    // finite: the first key group of a wavefront's step 0 ...
+      if (m_new == -INFINITY) return;                          // ... unless this wavefront has no key in this step
+      const float alpha = __expf(m_run - m_new);               // m_run = -inf -> 0
+      l_run *= alpha;
 #pragma unroll
-    for (int j = 0; j < EPC; ++j) acc[j] = 0.f;
+      for (int j = 0; j < EPC; ++j) acc[j] *= alpha;
+      m_run = m_new;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int kk = (i * 4 + wave) * KPL + sub;
-      const float p = __shfl(pv, kk < nk ? kk : 0);
-      if (kk < nk) {
-        const uint32x4 w = vr[i];
-        if (sizeof(T) == 2) {
-          acc[0] += p * bf16_lo(w.x); acc[1 % EPC] += p * bf16_hi(w.x);
-          acc[2 % EPC] += p * bf16_lo(w.y); acc[3 % EPC] += p * bf16_hi(w.y);
-          acc[4 % EPC] += p * bf16_lo(w.z); acc[5 % EPC] += p * bf16_hi(w.z);
-          acc[6 % EPC] += p * bf16_lo(w.w); acc[7 % EPC] += p * bf16_hi(w.w);
-        } else {
-          acc[0] += p * __uint_as_float(w.x); acc[1] += p * __uint_as_float(w.y);
-          acc[2] += p * __uint_as_float(w.z); acc[3] += p * __uint_as_float(w.w);
-        }
+      for (int i = 0; i < NI; ++i) {
+        const float pr = __expf(sc[i] - m_new);                // masked -> 0
+        l_run += pr;
+        float vf[EPC];
+        kvrow<T>::get(vr[buf][i], vf);
+#pragma unroll
+        for (int j = 0; j < EPC; ++j) acc[j] = fmaf(pr, vf[j], acc[j]);
       }
+    };
+    int base = 0;
+    for (; base + 2 * STEP < nk + STEP; base += 2 * STEP) {    // steps base and base + STEP both exist
+      request(1, base + STEP);
+      reduce(0, base);
+      if (base + 2 * STEP < nk) request(0, base + 2 * STEP);
+      reduce(1, base + STEP);
     }
-#pragma unroll
-    for (int j = 0; j < EPC; ++j)
-#pragma unroll
-      for (int o = 32; o >= LPK; o >>= 1) acc[j] += __shfl_xor(acc[j], o);
-    if (lane < LPK)
-#pragma unroll
-      for (int j = 0; j < EPC; ++j) part[wave][el + j] = acc[j];
-    __syncthreads();
-    for (int e = tid; e < DH; e += 256) wout[2 + e] = (part[0][e] + part[1][e]) + (part[2][e] + part[3][e]);
-    if (tid == 0) { wout[0] = m; wout[1] = l; }
+    if (base < nk) reduce(0, base);
   }
-
+  // ---- key subgroups of a wavefront, then the four wavefronts
+#pragma unroll
+  for (int o = 32; o >= LPK; o >>= 1) {
+    l_run += __shfl_xor(l_run, o);
+#pragma unroll
+    for (int j = 0; j < EPC; ++j) acc[j] += __shfl_xor(acc[j], o);
+  }
+  if (lane < LPK) {
+#pragma unroll
+    for (int j = 0; j < EPC; ++j) part[wave][el + j] = acc[j];
+  }
+  if (lane == 0) { stat[wave][0] = m_run; stat[wave][1] = l_run; }
+  __syncthreads();
+  const float m0 = stat[0][0], m1 = stat[1][0], m2 = stat[2][0], m3 = stat[3][0];
+  const float mm = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
+  const bool any = mm != -INFINITY;
+  const float f0 = any ? __expf(m0 - mm) : 0.f, f1 = any ? __expf(m1 - mm) : 0.f;
+  const float f2 = any ? __expf(m2 - mm) : 0.f, f3 = any ? __expf(m3 - mm) : 0.f;
+  const float lt = (f0 * stat[0][1] + f1 * stat[1][1]) + (f2 * stat[2][1] + f3 * stat[3][1]);
+  float* wout = work + (bh * S + split) * (DH + DEC_PAD);
+  for (int e = tid; e < DH; e += 256) {
+    const float v = (f0 * part[0][e] + f1 * part[1][e]) + (f2 * part[2][e] + f3 * part[3][e]);
+    if (S == 1 && out) store_as(out, (int64_t)b * ld_out + h * DH + e, lt > 0.f ? v / lt : 0.f, out_dtype);
+    else wout[DEC_PAD + e] = v;
+  }
+  if (!(S == 1 && out) && tid == 0) { wout[0] = mm; wout[1] = lt; }
 }
 
-// Grid (H, B): merge the partials of the non-empty splits.
+// Merge of the S partials of one (sequence, head), four elements per thread (the out-projection GEMV does the same
+// while it stages its input).
 template <int DH>
-__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ work, const int32_t* __restrict__ pos,
-                                                           int S, int H, int Tcap, void* __restrict__ out, int64_t ld_out,
-                                                           int out_dtype) {
-  __shared__ float wgt[64];
+__global__ __launch_bounds__(DH / 4) void attn_combine_kernel(const float* __restrict__ work, int S, int H,
+                                                              void* __restrict__ out, int64_t ld_out, int out_dtype) {
   const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int64_t bh = (int64_t)b * H + h;
-  const int nvalid = (pos[b] + 1 < Tcap) ? pos[b] + 1 : Tcap;
-  const int ns = (nvalid + DEC_CHUNK - 1) / DEC_CHUNK;    // non-empty splits (<= S <= 64)
-  const float* wb = work + bh * S * (DH + 2);
-  // The partial vectors do not depend on the weights: thread e requests element e of the first 16 partials before
-  // the barrier behind which the weights are visible, so the merge costs one memory round trip after the weights'
-  // own, not one per four splits.  (d_head <= 256: one element per thread.)
-  static_assert(DH <= 256, "one element per thread");
-  constexpr int G = 16;
-  const int e = tid;
-  float pv[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const int s2 = g < ns ? g : ns - 1;                      // beyond the last split: a valid address, weight 0 below
-    pv[g] = (e < DH) ? wb[(int64_t)s2 * (DH + 2) + 2 + e] : 0.f;
-  }
-  if (tid < 64) {
-    const float ms = (tid < ns) ? wb[(int64_t)tid * (DH + 2)] : -INFINITY;
-    const float ls = (tid < ns) ? wb[(int64_t)tid * (DH + 2) + 1] : 0.f;
-    const float mm = wave_max(ms);
-    const float f = (tid < ns) ? expf(ms - mm) : 0.f;
-    const float lt = wave_sum(f * ls);
-    wgt[tid] = f / lt;
-  }
-  __syncthreads();
-  if (e < DH) {
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    for (int s0 = 0; s0 < ns; s0 += G) {
-      if (s0 > 0) {
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-          const int s2 = s0 + g < ns ? s0 + g : ns - 1;
-          pv[g] = wb[(int64_t)s2 * (DH + 2) + 2 + e];
-        }
-      }
-#pragma unroll
-      for (int g = 0; g < G; g += 4) {
-        a0 += (s0 + g < ns ? wgt[s0 + g] : 0.f) * pv[g];
-        a1 += (s0 + g + 1 < ns ? wgt[s0 + g + 1] : 0.f) * pv[g + 1];
-        a2 += (s0 + g + 2 < ns ? wgt[s0 + g + 2] : 0.f) * pv[g + 2];
-        a3 += (s0 + g + 3 < ns ? wgt[s0 + g + 3] : 0.f) * pv[g + 3];
-      }
-    }
-    store_as(out, (int64_t)b * ld_out + h * DH + e, (a0 + a1) + (a2 + a3), out_dtype);
-  }
+  const floatx4 a = mtj_merge_partials(work + bh * S * (DH + DEC_PAD), S, DH, 4 * tid);
+  const int64_t o = (int64_t)b * ld_out + h * DH + 4 * tid;
+  store_as(out, o, a.x, out_dtype);
+  store_as(out, o + 1, a.y, out_dtype);
+  store_as(out, o + 2, a.z, out_dtype);
+  store_as(out, o + 3, a.w, out_dtype);
 }
 
-int decode_splits(int64_t Tcap) { return (int)((Tcap + DEC_CHUNK - 1) / DEC_CHUNK); }
+// key ranges per (sequence, head): about one workgroup per CU when the batch alone does not fill the chip; a range
+// never starts out shorter than 16 keys at the full window
+int decode_splits(int64_t B, int64_t H, int64_t Tcap) {
+  int64_t S = 256 / (B * H);
+  if (S > (Tcap + 15) / 16) S = (Tcap + 15) / 16;
+  if (S > MTJ_DEC_MAXS) S = MTJ_DEC_MAXS;
+  if (S < 1) S = 1;
+  return (int)S;
+}
 
 }  // namespace
 
@@ -494,7 +536,8 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
   MTJ_REQUIRE(B > 0 && H > 0 && Tp > 0 && Tp <= Tcap && ld_out >= H * dh && B < 65536 && H < 65536, MTJ_EINVAL,
               "mtj_attn_prefill: bad shape B=%lld H=%lld Tp=%lld Tcap=%lld", (long long)B, (long long)H,
               (long long)Tp, (long long)Tcap);
-  const int esz = dtype == MTJ_BF16 ? 2 : 4;
+  MTJ_REQUIRE(mtj_is_dtype(dtype), MTJ_EDTYPE, "mtj_attn_prefill: dtype %d", dtype);
+  const int esz = mtj_elem_size(dtype);
   MTJ_REQUIRE(ldvt >= (Tp + 63) / 64 * 64 && (ldvt * esz) % 16 == 0 && (ld_out * esz) % 16 == 0, MTJ_EALIGN,
               "mtj_attn_prefill: ldvt must be >= Tp rounded up to a multiple of 64, rows 16-byte aligned");
   MTJ_REQUIRE(mtj_aligned16(q) && mtj_aligned16(k_cache) && mtj_aligned16(v_t) && mtj_aligned16(out), MTJ_EALIGN,
@@ -514,6 +557,8 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
   } while (0)
   if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL(bf16_t, 256, 4, 32);
   else if (dtype == MTJ_BF16 && dh == 64) MTJ_PREFILL(bf16_t, 64, 8, 64);
+  else if (dtype == MTJ_F16 && dh == 256) MTJ_PREFILL(f16_t, 256, 4, 32);
+  else if (dtype == MTJ_F16 && dh == 64) MTJ_PREFILL(f16_t, 64, 8, 64);
   else if (dtype == MTJ_F32 && dh == 256) MTJ_PREFILL(float, 256, 4, 32);
   else if (dtype == MTJ_F32 && dh == 64) MTJ_PREFILL(float, 64, 4, 32);
   else return mtj_fail(MTJ_EINVAL, "mtj_attn_prefill: unsupported dtype %d / d_head %lld (64 or 256)", dtype, (long long)dh);
@@ -521,34 +566,46 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
   return mtj_check_launch("mtj_attn_prefill");
 }
 
+extern "C" int mtj_attn_decode_splits(int64_t B, int64_t H, int64_t Tcap) {
+  if (B <= 0 || H <= 0 || Tcap <= 0) return 0;
+  return decode_splits(B, H, Tcap);
+}
+
 extern "C" int64_t mtj_attn_decode_work_bytes(int64_t B, int64_t H, int64_t dh, int64_t Tcap) {
-  return B * H * (int64_t)decode_splits(Tcap) * (dh + 2) * (int64_t)sizeof(float);
+  if (B <= 0 || H <= 0 || Tcap <= 0 || dh <= 0) return 0;
+  return B * H * (int64_t)decode_splits(B, H, Tcap) * (dh + DEC_PAD) * (int64_t)sizeof(float);
 }
 
 namespace {
 
+// merge = false: only the partials are produced (the caller merges them, see mtj_attn_merge), out may be NULL
 int attn_decode_impl(const char* who, const float* q, const void* k_cache, const void* v_cache, const int32_t* pos,
                      int64_t B, int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
-                     void* work, void* stream) {
-  MTJ_REQUIRE(q && k_cache && v_cache && pos && out && work, MTJ_EINVAL, "%s: null pointer", who);
-  MTJ_REQUIRE(B > 0 && H > 0 && Tcap > 0 && ld_out >= H * dh && B < 65536 && H < 65536, MTJ_EINVAL, "%s: bad shape", who);
-  MTJ_REQUIRE(out_dtype == MTJ_F32 || out_dtype == MTJ_BF16, MTJ_EDTYPE, "%s: out_dtype %d", who, out_dtype);
+                     void* work, bool merge, void* stream) {
+  MTJ_REQUIRE(q && k_cache && v_cache && pos && work && (out || !merge), MTJ_EINVAL, "%s: null pointer", who);
+  MTJ_REQUIRE(B > 0 && H > 0 && Tcap > 0 && B < 65536 && H < 65536 && Tcap < (1ll << 30), MTJ_EINVAL, "%s: bad shape", who);
   MTJ_REQUIRE(mtj_aligned16(q) && mtj_aligned16(k_cache) && mtj_aligned16(v_cache) && mtj_aligned16(work), MTJ_EALIGN,
               "%s: pointers must be 16-byte aligned", who);
-  const int S = decode_splits(Tcap);
-  MTJ_REQUIRE(S <= 64, MTJ_ELIMIT, "%s: window of %lld slots exceeds %d", who, (long long)Tcap, 64 * DEC_CHUNK);
+  if (merge) {
+    MTJ_REQUIRE(ld_out >= H * dh, MTJ_EINVAL, "%s: ld_out < H * dh", who);
+    MTJ_REQUIRE(mtj_is_dtype(out_dtype), MTJ_EDTYPE, "%s: out_dtype %d", who, out_dtype);
+  }
+  const int S = decode_splits(B, H, Tcap);
   float* partials = reinterpret_cast<float*>(work);
   dim3 grid((unsigned)S, (unsigned)H, (unsigned)B);
   hipStream_t s = (hipStream_t)stream;
 #define MTJ_DECODE(T, DH)                                                                                         \
   do {                                                                                                            \
     attn_decode_kernel<T, DH><<<grid, 256, 0, s>>>(q, (const T*)k_cache, (const T*)v_cache, pos, (int)H, (int)Tcap, \
-                                                   partials);                                                     \
-    attn_combine_kernel<DH><<<dim3((unsigned)H, (unsigned)B), 256, 0, s>>>(partials, pos, S, (int)H, (int)Tcap, out, \
-                                                                           ld_out, out_dtype);                    \
+                                                   partials, out, ld_out, out_dtype);                             \
+    if (merge && S > 1)                                                                                           \
+      attn_combine_kernel<DH><<<dim3((unsigned)H, (unsigned)B), DH / 4, 0, s>>>(partials, S, (int)H, out, ld_out,  \
+                                                                                 out_dtype);                      \
   } while (0)
   if (dtype == MTJ_BF16 && dh == 256) MTJ_DECODE(bf16_t, 256);
   else if (dtype == MTJ_BF16 && dh == 64) MTJ_DECODE(bf16_t, 64);
+  else if (dtype == MTJ_F16 && dh == 256) MTJ_DECODE(f16_t, 256);
+  else if (dtype == MTJ_F16 && dh == 64) MTJ_DECODE(f16_t, 64);
   else if (dtype == MTJ_F32 && dh == 256) MTJ_DECODE(float, 256);
   else if (dtype == MTJ_F32 && dh == 64) MTJ_DECODE(float, 64);
   else return mtj_fail(MTJ_EINVAL, "%s: unsupported dtype %d / d_head %lld (64 or 256)", who, dtype, (long long)dh);
@@ -562,11 +619,26 @@ extern "C" int mtj_attn_decode(const float* q, const void* k_cache, const void* 
                                int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out, int out_dtype, int dtype,
                                void* work, void* stream) {
   return attn_decode_impl("mtj_attn_decode", q, k_cache, v_cache, pos, B, H, Tcap, dh, out, ld_out, out_dtype, dtype, work,
-                          stream);
+                          true, stream);
+}
+
+extern "C" int mtj_attn_decode_partials(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos,
+                                        int64_t B, int64_t H, int64_t Tcap, int64_t dh, int dtype, void* work,
+                                        mtj_attn_merge* merge, void* stream) {
+  MTJ_REQUIRE(merge, MTJ_EINVAL, "mtj_attn_decode_partials: null pointer");
+  const int rc = attn_decode_impl("mtj_attn_decode_partials", q, k_cache, v_cache, pos, B, H, Tcap, dh, nullptr, 0, MTJ_F32,
+                                  dtype, work, false, stream);
+  if (rc) return rc;
+  const int S = decode_splits(B, H, Tcap);
+  merge->partials = reinterpret_cast<const float*>(work);
+  merge->n_heads = (int32_t)H;
+  merge->d_head = (int32_t)dh;
+  merge->splits = S;
+  return MTJ_OK;
 }
 
 // ------------------------------------------------------------------------------------------------
-// The same two launches with the partial results kept in a device array that lives in the code object, for
+// The same launches with the partial results kept in a device array that lives in the code object, for
 // callers that cannot allocate (or pass) a workspace.  Every device that loads the library holds its own copy of
 // `scratch` at its own address: the address is looked up once per device (hipGetSymbolAddress with that device
 // current) and that pointer, never the array's name, is what host code hands to the kernels.  Nothing in
@@ -611,5 +683,5 @@ extern "C" int mtj_attn_decode_static(const float* q, const void* k_cache, const
   void* work = nullptr;
   if (int rc = scratch_address(&work)) return rc;
   return attn_decode_impl("mtj_attn_decode_static", q, k_cache, v_cache, pos, B, H, Tcap, dh, out, ld_out, out_dtype,
-                          dtype, work, stream);
+                          dtype, work, true, stream);
 }

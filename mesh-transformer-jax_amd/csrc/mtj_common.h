@@ -11,6 +11,9 @@
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16_t;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t uint32x4 __attribute__((ext_vector_type(4)));
@@ -80,6 +83,35 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, r);
 }
 
+// float32 -> float16, round to nearest even, saturating at the largest finite value instead of overflowing to inf
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  const f16_t h = (f16_t)__builtin_amdgcn_fmed3f(f, -65504.f, 65504.f);
+  return (uint32_t)__builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  const f16x2 r = {(f16_t)__builtin_amdgcn_fmed3f(lo, -65504.f, 65504.f), (f16_t)__builtin_amdgcn_fmed3f(hi, -65504.f, 65504.f)};
+  return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ float f16_lo(uint32_t packed) { return (float)__builtin_bit_cast(f16x2, packed).x; }
+__device__ __forceinline__ float f16_hi(uint32_t packed) { return (float)__builtin_bit_cast(f16x2, packed).y; }
+// two floats -> one 32-bit word of two 16-bit elements of run-time type dtype (MTJ_BF16 or MTJ_F16)
+__device__ __forceinline__ uint32_t pack_16x2(float lo, float hi, int dtype) {
+  return dtype == MTJ_F16 ? pack_f16x2(lo, hi) : pack_bf16x2(lo, hi);
+}
+// the same with the type known at compile time
+template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float lo, float hi) { return pack_bf16x2(lo, hi); }
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float lo, float hi) { return pack_f16x2(lo, hi); }
+template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t w);
+template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w);
+template <> __device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t w) { return bf16_lo(w); }
+template <> __device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t w) { return bf16_hi(w); }
+template <> __device__ __forceinline__ float unpack_lo<f16_t>(uint32_t w) { return f16_lo(w); }
+template <> __device__ __forceinline__ float unpack_hi<f16_t>(uint32_t w) { return f16_hi(w); }
+
+static inline int mtj_elem_size(int dtype) { return dtype == MTJ_F32 ? 4 : 2; }
+static inline bool mtj_is_dtype(int dtype) { return dtype == MTJ_F32 || dtype == MTJ_BF16 || dtype == MTJ_F16; }
+
 template <typename T> struct elem;
 template <> struct elem<float> {
   static constexpr int dtype = MTJ_F32;
@@ -96,9 +128,18 @@ template <> struct elem<bf16_t> {
   }
 };
 
+template <> struct elem<f16_t> {
+  static constexpr int dtype = MTJ_F16;
+  __device__ static __forceinline__ float load(const f16_t* p) { return (float)*p; }
+  __device__ static __forceinline__ void store(f16_t* p, float v) {
+    *reinterpret_cast<uint16_t*>(p) = (uint16_t)f32_to_f16_bits(v);
+  }
+};
+
 // store a float into a buffer whose element type is only known at run time
 __device__ __forceinline__ void store_as(void* base, int64_t idx, float v, int dtype) {
   if (dtype == MTJ_F32) reinterpret_cast<float*>(base)[idx] = v;
+  else if (dtype == MTJ_F16) reinterpret_cast<uint16_t*>(base)[idx] = (uint16_t)f32_to_f16_bits(v);
   else reinterpret_cast<uint16_t*>(base)[idx] = (uint16_t)f32_to_bf16_bits(v);
 }
 
@@ -111,6 +152,40 @@ __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
   return v;
+}
+
+// ---------------------------------------------------------------- merge of one-token attention partials
+// Partials of one (sequence, head): wb[s * (dh + MTJ_DEC_PAD)] = {max, sum, -, -, V[dh]} for key range s < S <= 8.
+// Returns elements e .. e+3 of sum_s exp(max_s - max) V_s / sum_s exp(max_s - max) sum_s.  Every load is issued
+// before the first is used and none depends on another; ranges beyond S read range S-1 again with weight 0.
+constexpr int MTJ_DEC_MAXS = 8;
+constexpr int MTJ_DEC_PAD = 4;
+__device__ __forceinline__ floatx4 mtj_merge_partials(const float* __restrict__ wb, int S, int dh, int e) {
+  float m[MTJ_DEC_MAXS], l[MTJ_DEC_MAXS];
+  floatx4 v[MTJ_DEC_MAXS];
+#pragma unroll
+  for (int s = 0; s < MTJ_DEC_MAXS; ++s) {
+    const float* p = wb + (int64_t)(s < S ? s : S - 1) * (dh + MTJ_DEC_PAD);
+    m[s] = p[0];
+    l[s] = p[1];
+    v[s] = *reinterpret_cast<const floatx4*>(p + MTJ_DEC_PAD + e);
+  }
+  float mm = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < MTJ_DEC_MAXS; ++s) {
+    if (s >= S) m[s] = -INFINITY;
+    mm = fmaxf(mm, m[s]);
+  }
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  float lt = 0.f;
+#pragma unroll
+  for (int s = 0; s < MTJ_DEC_MAXS; ++s) {
+    const float f = (m[s] == -INFINITY) ? 0.f : __expf(m[s] - mm);    // an empty range has max -inf
+    lt = fmaf(f, l[s], lt);
+    acc += f * v[s];
+  }
+  const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+  return acc * inv;
 }
 
 // jax.nn.gelu(approximate=True): 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3).
@@ -171,8 +246,8 @@ __device__ __forceinline__ inproj_pre inproj_prepare(const mtj_inproj& ip, const
   return p;
 }
 
-__device__ __forceinline__ void inproj_finish(const mtj_inproj& ip, int kv_dtype, const inproj_pre& p, float own,
-                                              float partner) {
+__device__ __forceinline__ void inproj_finish(const mtj_inproj& ip, const inproj_pre& p, float own, float partner) {
+  const int kv_dtype = ip.kv_dtype;
   if (p.kind < 0) return;
   if (p.kind == 3) {
     store_as(ip.act, p.idx, gelu_tanh(own + p.bias), ip.act_dtype);
@@ -187,7 +262,7 @@ __device__ __forceinline__ void inproj_finish(const mtj_inproj& ip, int kv_dtype
   }
 }
 
-__device__ __forceinline__ void inproj_store(const mtj_inproj& ip, const float* __restrict__ b1, int kv_dtype,
-                                             int64_t m, int64_t n, float own, float partner) {
-  inproj_finish(ip, kv_dtype, inproj_prepare(ip, b1, m, n), own, partner);
+__device__ __forceinline__ void inproj_store(const mtj_inproj& ip, const float* __restrict__ b1, int64_t m, int64_t n,
+                                             float own, float partner) {
+  inproj_finish(ip, inproj_prepare(ip, b1, m, n), own, partner);
 }

@@ -42,6 +42,50 @@ __global__ __launch_bounds__(256) void pack_kernel(const T* __restrict__ src, in
   }
 }
 
+// the same tiles with a change of type: dst = round(src * scale)
+template <typename TS, typename TD>
+__global__ __launch_bounds__(256) void pack_cvt_kernel(const TS* __restrict__ src, int64_t ld, int64_t K, int64_t N,
+                                                       TD* __restrict__ dst, int64_t Kt, int64_t n_off, int64_t k_off,
+                                                       float scale) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int64_t n0 = (int64_t)blockIdx.x * 32, k0 = (int64_t)blockIdx.y * 32;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t k = k0 + ty + i * 8, n = n0 + tx;
+    if (k < K && n < N) tile[ty + i * 8][tx] = elem<TS>::load(src + k * ld + n) * scale;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t n = n0 + ty + i * 8, k = k0 + tx;
+    if (k < K && n < N) elem<TD>::store(dst + (n_off + n) * Kt + k_off + k, tile[tx][ty + i * 8]);
+  }
+}
+
+extern "C" int mtj_pack_weight_cvt(const void* src, int64_t src_ld, int64_t K, int64_t N, void* dst, int64_t K_total,
+                                   int64_t n_off, int64_t k_off, int src_dtype, int dst_dtype, float scale, void* stream) {
+  MTJ_REQUIRE(src && dst, MTJ_EINVAL, "mtj_pack_weight_cvt: null pointer");
+  MTJ_REQUIRE(K > 0 && N > 0 && src_ld >= N && n_off >= 0 && k_off >= 0 && k_off + K <= K_total, MTJ_EINVAL,
+              "mtj_pack_weight_cvt: bad shape K=%lld N=%lld ld=%lld K_total=%lld k_off=%lld", (long long)K, (long long)N,
+              (long long)src_ld, (long long)K_total, (long long)k_off);
+  MTJ_REQUIRE(scale > 0.f && scale < INFINITY, MTJ_EINVAL, "mtj_pack_weight_cvt: scale must be positive and finite");
+  dim3 grid((unsigned)((N + 31) / 32), (unsigned)((K + 31) / 32));
+  hipStream_t s = (hipStream_t)stream;
+#define MTJ_CVT(SD, TS, DD, TD)                                                                                    \
+  if (src_dtype == SD && dst_dtype == DD) {                                                                        \
+    pack_cvt_kernel<TS, TD><<<grid, 256, 0, s>>>((const TS*)src, src_ld, K, N, (TD*)dst, K_total, n_off, k_off, scale); \
+    return mtj_check_launch("mtj_pack_weight_cvt");                                                               \
+  }
+  MTJ_CVT(MTJ_BF16, bf16_t, MTJ_F16, f16_t)
+  MTJ_CVT(MTJ_F32, float, MTJ_F16, f16_t)
+  MTJ_CVT(MTJ_F32, float, MTJ_BF16, bf16_t)
+  MTJ_CVT(MTJ_BF16, bf16_t, MTJ_F32, float)
+  MTJ_CVT(MTJ_F16, f16_t, MTJ_F32, float)
+#undef MTJ_CVT
+  return mtj_fail(MTJ_EDTYPE, "mtj_pack_weight_cvt: no conversion from dtype %d to dtype %d", src_dtype, dst_dtype);
+}
+
 extern "C" int mtj_pack_weight(const void* src, int64_t src_ld, int64_t K, int64_t N, void* dst, int64_t K_total,
                                int64_t n_off, int64_t k_off, int dtype, void* stream) {
   MTJ_REQUIRE(src && dst, MTJ_EINVAL, "mtj_pack_weight: null pointer");
@@ -52,7 +96,7 @@ extern "C" int mtj_pack_weight(const void* src, int64_t src_ld, int64_t K, int64
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MTJ_F32)
     pack_kernel<float><<<grid, 256, 0, s>>>((const float*)src, src_ld, K, N, (float*)dst, K_total, n_off, k_off);
-  else if (dtype == MTJ_BF16)
+  else if (dtype == MTJ_BF16 || dtype == MTJ_F16)
     pack_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)src, src_ld, K, N, (uint16_t*)dst, K_total, n_off, k_off);
   else
     return mtj_fail(MTJ_EDTYPE, "mtj_pack_weight: dtype %d", dtype);
@@ -82,6 +126,8 @@ extern "C" int mtj_embed(const int32_t* tok, int64_t M, const void* W, const flo
     embed_kernel<float><<<(unsigned)M, 256, 0, s>>>(tok, (const float*)W, b, n_vocab, d, out);
   else if (dtype == MTJ_BF16)
     embed_kernel<bf16_t><<<(unsigned)M, 256, 0, s>>>(tok, (const bf16_t*)W, b, n_vocab, d, out);
+  else if (dtype == MTJ_F16)
+    embed_kernel<f16_t><<<(unsigned)M, 256, 0, s>>>(tok, (const f16_t*)W, b, n_vocab, d, out);
   else
     return mtj_fail(MTJ_EDTYPE, "mtj_embed: dtype %d", dtype);
   return mtj_check_launch("mtj_embed");
@@ -90,7 +136,7 @@ extern "C" int mtj_embed(const int32_t* tok, int64_t M, const void* W, const flo
 // ---------------------------------------------------------------- LayerNorm: one wavefront per row
 // Two passes over a row that stays in registers (mean first, then centred variance, as the reference
 // computes jnp.var); all statistics float32.
-#define LN_MAX_PER_LANE 64  // d <= 64 * 64 * 4 = 16384
+#define LN_MAX_PER_LANE 64  // floats per lane: d <= 64 lanes * 64 = 4096
 
 template <int OUT_DTYPE>
 __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ scale,
@@ -133,8 +179,8 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const float* __restrict_
         *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(out) + row * d + 4 * c) = y;
       } else {
         uint32x2 p;
-        p.x = pack_bf16x2(y.x, y.y);
-        p.y = pack_bf16x2(y.z, y.w);
+        p.x = pack_16x2(y.x, y.y, OUT_DTYPE);
+        p.y = pack_16x2(y.z, y.w, OUT_DTYPE);
         *reinterpret_cast<uint32x2*>(reinterpret_cast<uint16_t*>(out) + row * d + 4 * c) = p;
       }
     }
@@ -154,6 +200,8 @@ extern "C" int mtj_layernorm(const float* x, const float* scale, const float* of
     layernorm_kernel<MTJ_F32><<<grid, 256, 0, s>>>(x, scale, offset, M, (int)d, out);
   else if (out_dtype == MTJ_BF16)
     layernorm_kernel<MTJ_BF16><<<grid, 256, 0, s>>>(x, scale, offset, M, (int)d, out);
+  else if (out_dtype == MTJ_F16)
+    layernorm_kernel<MTJ_F16><<<grid, 256, 0, s>>>(x, scale, offset, M, (int)d, out);
   else
     return mtj_fail(MTJ_EDTYPE, "mtj_layernorm: out_dtype %d", out_dtype);
   return mtj_check_launch("mtj_layernorm");

@@ -23,6 +23,18 @@ template <> struct mma<bf16_t> {
     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
   }
 };
+template <> struct mma<f16_t> {
+  static constexpr int EPC = 8;
+  struct frag { f16x8 v; };
+  __device__ static __forceinline__ frag load(const f16_t* p) {
+    frag f;
+    f.v = *reinterpret_cast<const f16x8*>(p);
+    return f;
+  }
+  __device__ static __forceinline__ void run(floatx16& c, const frag& a, const frag& b) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.v, b.v, c, 0, 0, 0);
+  }
+};
 template <> struct mma<float> {
   static constexpr int EPC = 4;
   struct frag { floatx4 lo, hi; };
@@ -53,17 +65,11 @@ struct gemm_args {
   void* out;
   int64_t ldo;
   int out_dtype;
-  int kv_dtype;
+  float alpha;            // multiplies the accumulator first (undoes a power-of-two scale of the packed weights)
   int splits;             // > 1: blockIdx.y owns a K range and stores a raw float32 partial at out + y * split_stride
   int64_t split_stride;
   mtj_inproj ip;
 };
-
-template <int DT>
-__device__ __forceinline__ void store_t(void* base, int64_t idx, float v) {
-  if (DT == MTJ_F32) reinterpret_cast<float*>(base)[idx] = v;
-  else reinterpret_cast<uint16_t*>(base)[idx] = (uint16_t)f32_to_bf16_bits(v);
-}
 
 // 16 consecutive elements, 16-byte vector stores (idx is a multiple of 16 elements, base 16-byte aligned)
 __device__ __forceinline__ void store16(void* base, int64_t idx, const float* v, int dtype) {
@@ -75,8 +81,8 @@ __device__ __forceinline__ void store16(void* base, int64_t idx, const float* v,
     uint32x4* p = reinterpret_cast<uint32x4*>(reinterpret_cast<uint16_t*>(base) + idx);
 #pragma unroll
     for (int q = 0; q < 2; ++q)
-      p[q] = uint32x4{pack_bf16x2(v[8 * q], v[8 * q + 1]), pack_bf16x2(v[8 * q + 2], v[8 * q + 3]),
-                      pack_bf16x2(v[8 * q + 4], v[8 * q + 5]), pack_bf16x2(v[8 * q + 6], v[8 * q + 7])};
+      p[q] = uint32x4{pack_16x2(v[8 * q], v[8 * q + 1], dtype), pack_16x2(v[8 * q + 2], v[8 * q + 3], dtype),
+                      pack_16x2(v[8 * q + 4], v[8 * q + 5], dtype), pack_16x2(v[8 * q + 6], v[8 * q + 7], dtype)};
   }
 }
 
@@ -174,7 +180,7 @@ __device__ __forceinline__ void epilogue(const gemm_args& a, void* out, floatx16
       if constexpr (nj < WN) nxt = load_ops(ni, nj);
       const col_info c = column(j);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) patch[(8 * (v / 4) + 4 * fg + (v % 4)) * PS + fr] = acc[i][j][v];
+      for (int v = 0; v < 16; ++v) patch[(8 * (v / 4) + 4 * fg + (v % 4)) * PS + fr] = acc[i][j][v] * a.alpha;
       __builtin_amdgcn_wave_barrier();
       float val[16];
 #pragma unroll
@@ -208,10 +214,10 @@ __device__ __forceinline__ void epilogue(const gemm_args& a, void* out, floatx16
               store16(a.ip.q, (bh * Tp + (m - b * Tp)) * dh + c.e0, val, a.ip.q_dtype);
             } else {
               const int slot = pos % a.ip.Tcap;
-              store16(c.seg == 1 ? a.ip.v_cache : a.ip.k_cache, (bh * a.ip.Tcap + slot) * dh + c.e0, val, a.kv_dtype);
+              store16(c.seg == 1 ? a.ip.v_cache : a.ip.k_cache, (bh * a.ip.Tcap + slot) * dh + c.e0, val, a.ip.kv_dtype);
               if (c.seg == 1 && a.ip.v_t && pos < a.ip.ldvt) {
 #pragma unroll
-                for (int k = 0; k < 16; ++k) store_as(a.ip.v_t, (bh * dh + c.e0 + k) * a.ip.ldvt + pos, val[k], a.kv_dtype);
+                for (int k = 0; k < 16; ++k) store_as(a.ip.v_t, (bh * dh + c.e0 + k) * a.ip.ldvt + pos, val[k], a.ip.kv_dtype);
               }
             }
           }
@@ -230,10 +236,9 @@ __device__ __forceinline__ void epilogue(const gemm_args& a, void* out, floatx16
         const int m = m0 + (wm * WM + i) * 32 + 8 * (v / 4) + 4 * fg + (v % 4);
         if (m < a.M && n_ok) {
           const int64_t idx = (int64_t)m * a.ldo + n;
-          const float val = acc[i][j][v] + bias;
+          const float val = acc[i][j][v] * a.alpha + bias;
           if (EPI == MTJ_EPI_RESID) reinterpret_cast<float*>(out)[idx] += val;
-          else if (a.out_dtype == MTJ_F32) reinterpret_cast<float*>(out)[idx] = val;
-          else reinterpret_cast<uint16_t*>(out)[idx] = (uint16_t)f32_to_bf16_bits(val);
+          else store_as(out, idx, val, a.out_dtype);
         }
       }
     });
@@ -407,9 +412,9 @@ constexpr int wait_lgkmcnt(int n) { return 0xf | (3 << 14) | (0x7 << 4) | ((n & 
 // are fetched under the last MFMAs of kt and the stage of kt is handed to the loads of kt+2.  Those eight
 // loads per wavefront are issued one per two MFMAs (a burst would stall the wavefront on the address queue
 // with its MFMAs behind it).  Rows beyond M or N are outside the buffer resource and read as zero.
-template <int EPI>
+template <typename T, int EPI>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
-  using T = bf16_t;
+  static_assert(sizeof(T) == 2, "16-bit operands");
   constexpr int WAVES_M = 2, WAVES_N = 4, WM = 4, WN = 2, NT = 512, BM = 256, BN = 256, BK = 64, NST = 2;
   constexpr int ROWB = BK * 2, CPR = BK / 8, OPB = BM * ROWB, STAGEB = 2 * OPB;
   constexpr int LOADS = BM * CPR / NT, ROWS_PER_LOAD = NT / CPR, KS = BK / 16;
@@ -478,13 +483,13 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) xo[ks] = ((2 * ks + fg) ^ swz(fr)) * 16;
   const int a_row = (wm * WM * 32 + fr) * ROWB, b_row = OPB + (wn * WN * 32 + fr) * ROWB;
-  bf16x8 fa[2][WM], fb[2][WN];
+  typename mma<T>::frag fa[2][WM], fb[2][WN];
   auto read_frags = [&](int st, int ks, int slot) {
     const unsigned char* p = smem + st * STAGEB + xo[ks];
 #pragma unroll
-    for (int i = 0; i < WM; ++i) fa[slot][i] = *reinterpret_cast<const bf16x8*>(p + a_row + i * 32 * ROWB);
+    for (int i = 0; i < WM; ++i) fa[slot][i] = mma<T>::load(reinterpret_cast<const T*>(p + a_row + i * 32 * ROWB));
 #pragma unroll
-    for (int j = 0; j < WN; ++j) fb[slot][j] = *reinterpret_cast<const bf16x8*>(p + b_row + j * 32 * ROWB);
+    for (int j = 0; j < WN; ++j) fb[slot][j] = mma<T>::load(reinterpret_cast<const T*>(p + b_row + j * 32 * ROWB));
   };
   if (KT > 1) __builtin_amdgcn_s_waitcnt(wait_vmcnt(2 * LOADS));
   else __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
@@ -514,7 +519,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
       __builtin_amdgcn_sched_barrier(0);
       for_stages<0, WM * WN>([&](auto Q_) {
         constexpr int q = decltype(Q_)::value, i = q / WN, j = q % WN;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+        mma<T>::run(acc[i][j], fa[cur][i], fb[cur][j]);
         if constexpr ((first_half || second_half) && (q & 1)) {
           __builtin_amdgcn_sched_barrier(0);
           if (go) issue_one(l_st, l_kt, std::integral_constant<int, (first_half ? 0 : LOADS) + q / 2>{});
@@ -533,13 +538,13 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
   epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, out, acc, smem, m0, n0);
 }
 
-template <int EPI>
+template <typename T, int EPI>
 int launch_dma(const gemm_args& a, hipStream_t s) {
   constexpr size_t lds = 2 * 2 * 256 * 64 * 2;
   static mtj_device_once once;
-  if (int rc = mtj_allow_lds(once, "mtj_gemm", &gemm_dma_kernel<EPI>, lds)) return rc;
+  if (int rc = mtj_allow_lds(once, "mtj_gemm", &gemm_dma_kernel<T, EPI>, lds)) return rc;
   const int tiles = ((a.M + 255) / 256) * ((a.N + 255) / 256);
-  gemm_dma_kernel<EPI><<<dim3(tiles, a.splits), 512, lds, s>>>(a);
+  gemm_dma_kernel<T, EPI><<<dim3(tiles, a.splits), 512, lds, s>>>(a);
   return mtj_check_launch("mtj_gemm");
 }
 
@@ -560,9 +565,10 @@ template <typename T, int EPI, int BK>
 int dispatch_tile(const gemm_args& a, hipStream_t s) {
   if (a.M <= 32) return launch<T, EPI, 1, 4, 1, 1, BK, 2>(a, s);    // 32 x 128: batched decode, weights stream once
   if (a.M <= 64) return launch<T, EPI, 1, 4, 2, 1, BK, 2>(a, s);    // 64 x 128
-  if constexpr (std::is_same<T, bf16_t>::value) {
+  if constexpr (sizeof(T) == 2) {
+    // e.g. M = 16384, N = 28672 or N = 4096 (a whole 6B layer at 8 x 2048 tokens): 7168 / 1024 tiles
     const int64_t big = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
-    if (big * a.splits >= 200) return launch_dma<EPI>(a, s);                         // 256 x 256, 8 wavefronts of 128 x 64
+    if (big * a.splits >= 200) return launch_dma<T, EPI>(a, s);                         // 256 x 256, 8 wavefronts of 128 x 64
   }
   return launch<T, EPI, 2, 2, 2, 2, BK, 2>(a, s);                   // 128 x 128
 }
@@ -600,9 +606,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     float* o = reinterpret_cast<float*>(out) + idx;
     o[0] = acc.x; o[1] = acc.y; o[2] = acc.z; o[3] = acc.w;
   } else {
-    uint16_t* o = reinterpret_cast<uint16_t*>(out) + idx;
-    o[0] = (uint16_t)f32_to_bf16_bits(acc.x); o[1] = (uint16_t)f32_to_bf16_bits(acc.y);
-    o[2] = (uint16_t)f32_to_bf16_bits(acc.z); o[3] = (uint16_t)f32_to_bf16_bits(acc.w);
+    uint32x2 pk;
+    pk.x = pack_16x2(acc.x, acc.y, out_dtype);
+    pk.y = pack_16x2(acc.z, acc.w, out_dtype);
+    *reinterpret_cast<uint32x2*>(reinterpret_cast<uint16_t*>(out) + idx) = pk;
   }
 }
 
@@ -679,8 +686,8 @@ __global__ __launch_bounds__(1024) void splitk_reduce_ln_kernel(const float* __r
         *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(h) + (int64_t)m * ldh + n) = y;
       } else {
         uint32x2 pk;
-        pk.x = pack_bf16x2(y.x, y.y);
-        pk.y = pack_bf16x2(y.z, y.w);
+        pk.x = pack_16x2(y.x, y.y, h_dtype);
+        pk.y = pack_16x2(y.z, y.w, h_dtype);
         *reinterpret_cast<uint32x2*>(reinterpret_cast<uint16_t*>(h) + (int64_t)m * ldh + n) = pk;
       }
     }
@@ -690,14 +697,14 @@ __global__ __launch_bounds__(1024) void splitk_reduce_ln_kernel(const float* __r
 // how many K ranges a skinny problem is cut into so that its few output tiles still fill the chip
 int pick_splits(int64_t M, int64_t N, int64_t K, int dtype) {
   if (N % 4) return 1;
-  const int bk = dtype == MTJ_BF16 ? 64 : 32;
+  const int bk = dtype == MTJ_F32 ? 32 : 64;
   const int64_t kt = K / bk;
   int splits = 1;
   if (M <= 64) {          // one row of 32 x 128 or 64 x 128 tiles: up to 16 ranges
     const int64_t tiles = (N + 127) / 128;
     while (splits < 16 && tiles * splits * 2 <= 256 && kt % (splits * 2) == 0 && kt / (splits * 2) >= 4) splits *= 2;
   } else {
-    if (dtype == MTJ_BF16) {   // 256 x 256 tiles of the direct-to-LDS kernel, one workgroup per CU (a short prompt's out projection)
+    if (dtype != MTJ_F32) {   // 256 x 256 tiles of the direct-to-LDS kernel, one workgroup per CU (a short prompt's out projection)
       const int64_t big = ((M + 255) / 256) * ((N + 255) / 256);
       while (splits < 16 && big * splits * 2 <= 256 && kt % (splits * 2) == 0 && kt / (splits * 2) >= 16) splits *= 2;
       if (big * splits >= 200) return splits;
@@ -712,9 +719,9 @@ int pick_splits(int64_t M, int64_t N, int64_t K, int dtype) {
 
 int check_common(const void* A, int64_t lda, const void* W, int64_t M, int64_t N, int64_t K, int dtype, const char* who) {
   MTJ_REQUIRE(A && W, MTJ_EINVAL, "%s: null pointer", who);
-  MTJ_REQUIRE(dtype == MTJ_F32 || dtype == MTJ_BF16, MTJ_EDTYPE, "%s: dtype %d", who, dtype);
-  const int bk = dtype == MTJ_BF16 ? 64 : 32;
-  const int esz = dtype == MTJ_BF16 ? 2 : 4;
+  MTJ_REQUIRE(mtj_is_dtype(dtype), MTJ_EDTYPE, "%s: dtype %d", who, dtype);
+  const int bk = dtype == MTJ_F32 ? 32 : 64;
+  const int esz = mtj_elem_size(dtype);
   MTJ_REQUIRE(M > 0 && N > 0 && K > 0 && K % bk == 0 && lda >= K, MTJ_EINVAL,
               "%s: bad shape M=%lld N=%lld K=%lld lda=%lld (K must be a multiple of %d)", who, (long long)M,
               (long long)N, (long long)K, (long long)lda, bk);
@@ -728,13 +735,21 @@ int check_common(const void* A, int64_t lda, const void* W, int64_t M, int64_t N
 
 }  // namespace
 
+namespace {
+int dispatch_dtype(const gemm_args& a, int dtype, int epi, hipStream_t s) {
+  if (dtype == MTJ_BF16) return dispatch<bf16_t, 64>(a, epi, s);
+  if (dtype == MTJ_F16) return dispatch<f16_t, 64>(a, epi, s);
+  return dispatch<float, 32>(a, epi, s);
+}
+}  // namespace
+
 extern "C" int mtj_gemm(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
-                        int dtype, int epi, void* out, int64_t ldo, int out_dtype, const mtj_inproj* ip,
+                        int dtype, int epi, void* out, int64_t ldo, int out_dtype, const mtj_inproj* ip, float alpha,
                         void* stream) {
   if (int rc = check_common(A, lda, W, M, N, K, dtype, "mtj_gemm")) return rc;
   gemm_args a{};
   a.A = A; a.lda = lda; a.W = W; a.bias = bias; a.M = (int)M; a.N = (int)N; a.K = (int)K;
-  a.out = out; a.ldo = ldo; a.out_dtype = out_dtype; a.kv_dtype = dtype; a.splits = 1;
+  a.out = out; a.ldo = ldo; a.out_dtype = out_dtype; a.alpha = alpha; a.splits = 1;
   if (epi == MTJ_EPI_INPROJ) {
     MTJ_REQUIRE(ip && bias, MTJ_EINVAL, "mtj_gemm: INPROJ needs ip and the fc_in bias");
     a.ip = *ip;
@@ -743,49 +758,45 @@ extern "C" int mtj_gemm(const void* A, int64_t lda, const void* W, const float* 
                     ip->rotary_dims % 16 == 0 && ip->ld_act % 16 == 0 &&
                     ip->rotary_dims <= ip->d_head && ip->Tcap > 0 && ip->max_pos > 0 && ip->pos0 && ip->sin_tab &&
                     ip->cos_tab && ip->q && ip->k_cache && ip->v_cache && ip->act && ip->ld_act >= N - 2 * d &&
-                    (ip->act_dtype == MTJ_F32 || ip->act_dtype == MTJ_BF16) &&
-                    (ip->q_dtype == MTJ_F32 || ip->q_dtype == MTJ_BF16) && (!ip->v_t || ip->ldvt >= ip->Tp),
+                    mtj_is_dtype(ip->act_dtype) && mtj_is_dtype(ip->q_dtype) && mtj_is_dtype(ip->kv_dtype) &&
+                    (!ip->v_t || ip->ldvt >= ip->Tp),
                 MTJ_EINVAL, "mtj_gemm: inconsistent INPROJ geometry");
     MTJ_REQUIRE(mtj_aligned16(bias) && mtj_aligned16(ip->sin_tab) && mtj_aligned16(ip->cos_tab), MTJ_EALIGN,
                 "mtj_gemm: the fc_in bias and the rotary tables must be 16-byte aligned");
   } else if (epi == MTJ_EPI_STORE) {
-    MTJ_REQUIRE(out && ldo >= N && (out_dtype == MTJ_F32 || out_dtype == MTJ_BF16), MTJ_EINVAL,
-                "mtj_gemm: STORE needs out with ldo >= N");
+    MTJ_REQUIRE(out && ldo >= N && mtj_is_dtype(out_dtype), MTJ_EINVAL, "mtj_gemm: STORE needs out with ldo >= N");
   } else if (epi == MTJ_EPI_RESID) {
     MTJ_REQUIRE(out && ldo >= N, MTJ_EINVAL, "mtj_gemm: RESID needs out with ldo >= N");
   } else {
     return mtj_fail(MTJ_EINVAL, "mtj_gemm: epilogue %d", epi);
   }
-  hipStream_t s = (hipStream_t)stream;
-  return dtype == MTJ_BF16 ? dispatch<bf16_t, 64>(a, epi, s) : dispatch<float, 32>(a, epi, s);
+  return dispatch_dtype(a, dtype, epi, (hipStream_t)stream);
 }
 
 extern "C" int64_t mtj_gemm_splitk_work_bytes(int64_t M, int64_t N, int64_t K, int dtype) {
-  if (M <= 0 || N <= 0 || K <= 0 || (dtype != MTJ_F32 && dtype != MTJ_BF16)) return 0;
+  if (M <= 0 || N <= 0 || K <= 0 || !mtj_is_dtype(dtype)) return 0;
   const int splits = pick_splits(M, N, K, dtype);
   return splits > 1 ? (int64_t)splits * M * N * (int64_t)sizeof(float) : 0;
 }
 
 extern "C" int mtj_gemm_splitk(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N,
                                int64_t K, int dtype, int epi, void* out, int64_t ldo, int out_dtype, void* work,
-                               int64_t work_bytes, void* stream) {
+                               int64_t work_bytes, float alpha, void* stream) {
   MTJ_REQUIRE(epi == MTJ_EPI_STORE || epi == MTJ_EPI_RESID, MTJ_EINVAL, "mtj_gemm_splitk: epilogue %d", epi);
   if (int rc = check_common(A, lda, W, M, N, K, dtype, "mtj_gemm_splitk")) return rc;
   const int splits = pick_splits(M, N, K, dtype);
-  if (splits == 1) return mtj_gemm(A, lda, W, bias, M, N, K, dtype, epi, out, ldo, out_dtype, nullptr, stream);
+  if (splits == 1) return mtj_gemm(A, lda, W, bias, M, N, K, dtype, epi, out, ldo, out_dtype, nullptr, alpha, stream);
   MTJ_REQUIRE(out && ldo >= N && ldo % 4 == 0 && mtj_aligned16(out) && (!bias || mtj_aligned16(bias)), MTJ_EINVAL,
               "mtj_gemm_splitk: out needs ldo >= N, a multiple of 4, and 16-byte alignment (bias too)");
-  MTJ_REQUIRE(epi == MTJ_EPI_RESID || out_dtype == MTJ_F32 || out_dtype == MTJ_BF16, MTJ_EDTYPE,
-              "mtj_gemm_splitk: out_dtype %d", out_dtype);
+  MTJ_REQUIRE(epi == MTJ_EPI_RESID || mtj_is_dtype(out_dtype), MTJ_EDTYPE, "mtj_gemm_splitk: out_dtype %d", out_dtype);
   MTJ_REQUIRE(work && mtj_aligned16(work) && work_bytes >= (int64_t)splits * M * N * (int64_t)sizeof(float), MTJ_EINVAL,
               "mtj_gemm_splitk: work must hold mtj_gemm_splitk_work_bytes() bytes");
   gemm_args a{};
   a.A = A; a.lda = lda; a.W = W; a.bias = nullptr; a.M = (int)M; a.N = (int)N; a.K = (int)K;
-  a.out = work; a.ldo = N; a.out_dtype = MTJ_F32; a.kv_dtype = dtype;
+  a.out = work; a.ldo = N; a.out_dtype = MTJ_F32; a.alpha = alpha;
   a.splits = splits; a.split_stride = M * N;
   hipStream_t s = (hipStream_t)stream;
-  const int rc = dtype == MTJ_BF16 ? dispatch<bf16_t, 64>(a, MTJ_EPI_STORE, s) : dispatch<float, 32>(a, MTJ_EPI_STORE, s);
-  if (rc) return rc;
+  if (int rc = dispatch_dtype(a, dtype, MTJ_EPI_STORE, s)) return rc;
   const int64_t quads = M * (N / 4);
   const unsigned grid = (unsigned)((quads + 255) / 256);
   if (epi == MTJ_EPI_RESID)
@@ -798,9 +809,9 @@ extern "C" int mtj_gemm_splitk(const void* A, int64_t lda, const void* W, const 
 extern "C" int mtj_gemm_splitk_ln(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N,
                                   int64_t K, int dtype, float* x, int64_t ldx, void* work, int64_t work_bytes,
                                   const float* ln_scale, const float* ln_offset, void* h, int64_t ldh, int h_dtype,
-                                  void* stream) {
+                                  float alpha, void* stream) {
   MTJ_REQUIRE(ln_scale && ln_offset && h && x, MTJ_EINVAL, "mtj_gemm_splitk_ln: null pointer");
-  MTJ_REQUIRE(h_dtype == MTJ_F32 || h_dtype == MTJ_BF16, MTJ_EDTYPE, "mtj_gemm_splitk_ln: h_dtype %d", h_dtype);
+  MTJ_REQUIRE(mtj_is_dtype(h_dtype), MTJ_EDTYPE, "mtj_gemm_splitk_ln: h_dtype %d", h_dtype);
   MTJ_REQUIRE(N % 4 == 0 && N <= 4 * RLN_Q * 1024 && ldh >= N && ldh % 4 == 0 && ldx >= N && ldx % 4 == 0 &&
                   mtj_aligned16(x) && mtj_aligned16(h) && mtj_aligned16(ln_scale) && mtj_aligned16(ln_offset) &&
                   (!bias || mtj_aligned16(bias)),
@@ -809,18 +820,17 @@ extern "C" int mtj_gemm_splitk_ln(const void* A, int64_t lda, const void* W, con
   const int splits = pick_splits(M, N, K, dtype);
   hipStream_t s = (hipStream_t)stream;
   if (splits == 1) {      // no partials to reduce: the product with its own residual epilogue, then the plain LayerNorm
-    if (int rc = mtj_gemm(A, lda, W, bias, M, N, K, dtype, MTJ_EPI_RESID, x, ldx, MTJ_F32, nullptr, stream)) return rc;
     MTJ_REQUIRE(ldx == N && ldh == N, MTJ_EINVAL, "mtj_gemm_splitk_ln: without a split, x and h must be dense");
+    if (int rc = mtj_gemm(A, lda, W, bias, M, N, K, dtype, MTJ_EPI_RESID, x, ldx, MTJ_F32, nullptr, alpha, stream)) return rc;
     return mtj_layernorm(x, ln_scale, ln_offset, M, N, h, h_dtype, stream);
   }
   MTJ_REQUIRE(work && mtj_aligned16(work) && work_bytes >= (int64_t)splits * M * N * (int64_t)sizeof(float), MTJ_EINVAL,
               "mtj_gemm_splitk_ln: work must hold mtj_gemm_splitk_work_bytes() bytes");
   gemm_args a{};
   a.A = A; a.lda = lda; a.W = W; a.bias = nullptr; a.M = (int)M; a.N = (int)N; a.K = (int)K;
-  a.out = work; a.ldo = N; a.out_dtype = MTJ_F32; a.kv_dtype = dtype;
+  a.out = work; a.ldo = N; a.out_dtype = MTJ_F32; a.alpha = alpha;
   a.splits = splits; a.split_stride = M * N;
-  const int rc = dtype == MTJ_BF16 ? dispatch<bf16_t, 64>(a, MTJ_EPI_STORE, s) : dispatch<float, 32>(a, MTJ_EPI_STORE, s);
-  if (rc) return rc;
+  if (int rc = dispatch_dtype(a, dtype, MTJ_EPI_STORE, s)) return rc;
   splitk_reduce_ln_kernel<<<(unsigned)M, 1024, 0, s>>>((const float*)work, splits, M * N, (int)N, bias, x, ldx, ln_scale,
                                                        ln_offset, h, ldh, h_dtype);
   return mtj_check_launch("mtj_gemm_splitk_ln");

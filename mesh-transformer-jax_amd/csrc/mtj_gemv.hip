@@ -21,6 +21,21 @@ template <> struct chunk<bf16_t> {
     acc = fmaf(bf16_hi(w.w), x1.w, acc);
   }
 };
+template <> struct chunk<f16_t> {
+  static constexpr int EPC = 8;
+  __device__ static __forceinline__ void fma(const uint32x4& w, const float* __restrict__ xs, float& acc) {
+    const floatx4 x0 = *reinterpret_cast<const floatx4*>(xs);
+    const floatx4 x1 = *reinterpret_cast<const floatx4*>(xs + 4);
+    acc = fmaf(f16_lo(w.x), x0.x, acc);
+    acc = fmaf(f16_hi(w.x), x0.y, acc);
+    acc = fmaf(f16_lo(w.y), x0.z, acc);
+    acc = fmaf(f16_hi(w.y), x0.w, acc);
+    acc = fmaf(f16_lo(w.z), x1.x, acc);
+    acc = fmaf(f16_hi(w.z), x1.y, acc);
+    acc = fmaf(f16_lo(w.w), x1.z, acc);
+    acc = fmaf(f16_hi(w.w), x1.w, acc);
+  }
+};
 template <> struct chunk<float> {
   static constexpr int EPC = 4;
   __device__ static __forceinline__ void fma(const uint32x4& w, const float* __restrict__ xs, float& acc) {
@@ -42,8 +57,8 @@ struct gemv_args {
   int epi;
   void* out;
   int out_dtype;
-  int kv_dtype;
   mtj_inproj ip;
+  mtj_attn_merge am;      // partials == NULL: x is read as it is
 };
 
 // One workgroup of 16 wavefronts per CU, all resident at once (a second round of workgroups would pay the
@@ -59,7 +74,8 @@ struct gemv_args {
 // current one is consumed, so a wavefront never has an empty memory queue - and no load is conditional.  (Dealing
 // the rows out round-robin instead, so that the chip reads one contiguous window at a time, streams ~5 % faster in
 // a plain read but scatters every lane's epilogue loads and stores: 43.5 us against 40.2 for the 235 MB launch.)
-template <typename T, int U, bool FULL>
+// MERGE: the leading inputs are merged from one-token attention partials (a.am) instead of being read from x.
+template <typename T, int U, bool FULL, bool MERGE>
 __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   extern __shared__ __align__(16) float xs[];
   __shared__ float red[2][16];
@@ -155,7 +171,15 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
         xs[k] = (a.ln_scale[k] * inv) * (xs[k] - mean) + a.ln_offset[k];
     }
   } else {
-    for (int k = tid * 4; k < K; k += blockDim.x * 4)
+    // the leading H * dh inputs may come from the per-range partials of the one-token attention
+    const int dm = MERGE ? a.am.n_heads * a.am.d_head : 0;
+    if (MERGE)
+    for (int k = tid * 4; k < dm; k += blockDim.x * 4) {
+      const int h = k / a.am.d_head, e = k - h * a.am.d_head;
+      *reinterpret_cast<floatx4*>(xs + k) =
+          mtj_merge_partials(a.am.partials + (int64_t)h * a.am.splits * (a.am.d_head + MTJ_DEC_PAD), a.am.splits, a.am.d_head, e);
+    }
+    for (int k = dm + tid * 4; k < K; k += blockDim.x * 4)
       *reinterpret_cast<floatx4*>(xs + k) = *reinterpret_cast<const floatx4*>(a.x + k);
   }
   __syncthreads();
@@ -226,7 +250,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   // ---- epilogue: every lane finishes its own row
   if (pairs) {
     const float partner = __shfl_xor(mine, 1);
-    if (lane < nrows) inproj_finish(a.ip, a.kv_dtype, pre, mine, partner);
+    if (lane < nrows) inproj_finish(a.ip, pre, mine, partner);
   } else if (lane < nrows) {
     const int64_t n = row0 + lane;
     if (a.epi == MTJ_EPI_STORE) store_as(a.out, n, mine + pre_add, a.out_dtype);
@@ -234,7 +258,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   }
 }
 
-template <typename T, int U, bool FULL>
+template <typename T, int U, bool FULL, bool MERGE>
 int launch(const gemv_args& a, hipStream_t s) {
   const size_t lds = (size_t)a.K * sizeof(float);
   const int64_t units = a.epi == MTJ_EPI_INPROJ ? a.N / 2 : a.N;
@@ -244,23 +268,24 @@ int launch(const gemv_args& a, hipStream_t s) {
   const int64_t upw = a.epi == MTJ_EPI_INPROJ ? 2 : 1;
   while ((units + grid * 16 - 1) / (grid * 16) * upw > 62) grid *= 2;   // a lane per row: <= 64 rows per wavefront
   static mtj_device_once once;
-  if (int rc = mtj_allow_lds(once, "mtj_gemv", &gemv_kernel<T, U, FULL>, 160 * 1024 - 256)) return rc;
-  gemv_kernel<T, U, FULL><<<(unsigned)grid, 1024, lds, s>>>(a);
+  if (int rc = mtj_allow_lds(once, "mtj_gemv", &gemv_kernel<T, U, FULL, MERGE>, 160 * 1024 - 256)) return rc;
+  gemv_kernel<T, U, FULL, MERGE><<<(unsigned)grid, 1024, lds, s>>>(a);
   return mtj_check_launch("mtj_gemv");
 }
 
 template <typename T>
 int dispatch(const gemv_args& a, hipStream_t s) {
   constexpr int U = 8;
-  if (a.K % (U * 64 * chunk<T>::EPC) == 0) return launch<T, U, true>(a, s);
-  return launch<T, U, false>(a, s);
+  const bool full = a.K % (U * 64 * chunk<T>::EPC) == 0;
+  if (a.am.partials) return full ? launch<T, U, true, true>(a, s) : launch<T, U, false, true>(a, s);
+  return full ? launch<T, U, true, false>(a, s) : launch<T, U, false, false>(a, s);
 }
 
 }  // namespace
 
 extern "C" int mtj_gemv(const float* x, const float* ln_scale, const float* ln_offset, const void* W,
                         const float* bias, int64_t N, int64_t K, int dtype, int epi, void* out, int out_dtype,
-                        const mtj_inproj* ip, void* stream) {
+                        const mtj_inproj* ip, const mtj_attn_merge* am, void* stream) {
   MTJ_REQUIRE(x && W, MTJ_EINVAL, "mtj_gemv: null pointer");
   MTJ_REQUIRE(N > 0 && K > 0 && K % 8 == 0, MTJ_EINVAL, "mtj_gemv: K=%lld must be a positive multiple of 8", (long long)K);
   MTJ_REQUIRE(K * 4 <= 160 * 1024 - 512, MTJ_ELIMIT, "mtj_gemv: K=%lld floats do not fit LDS", (long long)K);
@@ -268,7 +293,7 @@ extern "C" int mtj_gemv(const float* x, const float* ln_scale, const float* ln_o
   MTJ_REQUIRE((ln_scale == nullptr) == (ln_offset == nullptr), MTJ_EINVAL, "mtj_gemv: ln_scale/ln_offset go together");
   gemv_args a{};
   a.x = x; a.ln_scale = ln_scale; a.ln_offset = ln_offset; a.W = W; a.bias = bias;
-  a.N = N; a.K = K; a.epi = epi; a.out = out; a.out_dtype = out_dtype; a.kv_dtype = dtype;
+  a.N = N; a.K = K; a.epi = epi; a.out = out; a.out_dtype = out_dtype;
   if (epi == MTJ_EPI_INPROJ) {
     MTJ_REQUIRE(ip && bias, MTJ_EINVAL, "mtj_gemv: INPROJ needs ip and the fc_in bias");
     a.ip = *ip;
@@ -276,19 +301,27 @@ extern "C" int mtj_gemv(const float* x, const float* ln_scale, const float* ln_o
     MTJ_REQUIRE(ip->Tp == 1 && N > 3 * d && N % 2 == 0 && ip->rotary_dims % 2 == 0 && ip->rotary_dims <= ip->d_head &&
                     ip->Tcap > 0 && ip->max_pos > 0 && ip->pos0 && ip->sin_tab && ip->cos_tab && ip->q && ip->k_cache &&
                     ip->v_cache && ip->act && ip->ld_act >= N - 2 * d &&
-                    (ip->act_dtype == MTJ_F32 || ip->act_dtype == MTJ_BF16) &&
-                    (ip->q_dtype == MTJ_F32 || ip->q_dtype == MTJ_BF16),
+                    mtj_is_dtype(ip->act_dtype) && mtj_is_dtype(ip->q_dtype) && mtj_is_dtype(ip->kv_dtype),
                 MTJ_EINVAL, "mtj_gemv: inconsistent INPROJ geometry");
     a.ip.v_t = nullptr;
   } else if (epi == MTJ_EPI_STORE) {
-    MTJ_REQUIRE(out && (out_dtype == MTJ_F32 || out_dtype == MTJ_BF16), MTJ_EINVAL, "mtj_gemv: STORE needs out");
+    MTJ_REQUIRE(out && mtj_is_dtype(out_dtype), MTJ_EINVAL, "mtj_gemv: STORE needs out");
   } else if (epi == MTJ_EPI_RESID) {
     MTJ_REQUIRE(out && out != (const void*)x, MTJ_EINVAL, "mtj_gemv: RESID needs out distinct from x");
   } else {
     return mtj_fail(MTJ_EINVAL, "mtj_gemv: epilogue %d", epi);
   }
+  if (am) {
+    const int64_t dm = (int64_t)am->n_heads * am->d_head;
+    MTJ_REQUIRE(!ln_scale && am->partials && mtj_aligned16(am->partials) && am->n_heads > 0 && am->d_head > 0 &&
+                    am->d_head % 4 == 0 && dm <= K && am->splits >= 1 && am->splits <= MTJ_DEC_MAXS,
+                MTJ_EINVAL, "mtj_gemv: attention partials need 1..%d ranges, d_head a multiple of 4, H*dh <= K and no LayerNorm",
+                MTJ_DEC_MAXS);
+    a.am = *am;
+  }
   hipStream_t s = (hipStream_t)stream;
   if (dtype == MTJ_F32) return dispatch<float>(a, s);
   if (dtype == MTJ_BF16) return dispatch<bf16_t>(a, s);
+  if (dtype == MTJ_F16) return dispatch<f16_t>(a, s);
   return mtj_fail(MTJ_EDTYPE, "mtj_gemv: dtype %d", dtype);
 }

@@ -7,9 +7,9 @@ raises, so a GPU run can never silently take another path.
 import ctypes as C
 import os
 
-F32, BF16 = 0, 1
+F32, BF16, F16 = 0, 1, 2
 EPI_STORE, EPI_RESID, EPI_INPROJ = 0, 1, 2
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmtj_hip.so")
 
@@ -22,10 +22,15 @@ class InProj(C.Structure):
         ("n_heads", C.c_int32), ("d_head", C.c_int32), ("rotary_dims", C.c_int32),
         ("Tp", C.c_int32), ("Tcap", C.c_int32), ("max_pos", C.c_int32),
         ("pos0", _p), ("sin_tab", _p), ("cos_tab", _p),
-        ("q", _p), ("q_dtype", C.c_int32),
+        ("q", _p), ("q_dtype", C.c_int32), ("kv_dtype", C.c_int32),
         ("k_cache", _p), ("v_cache", _p), ("v_t", _p), ("ldvt", _i64),
         ("act", _p), ("ld_act", _i64), ("act_dtype", C.c_int32),
     ]
+
+
+class AttnMerge(C.Structure):
+    """mtj_attn_merge"""
+    _fields_ = [("partials", _p), ("n_heads", C.c_int32), ("d_head", C.c_int32), ("splits", C.c_int32)]
 
 
 class NextEmbed(C.Structure):
@@ -38,16 +43,20 @@ SIGNATURES = {
     "mtj_version": (_i32, []),
     "mtj_last_error": (C.c_char_p, []),
     "mtj_pack_weight": (_i32, [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _i32, _p]),
+    "mtj_pack_weight_cvt": (_i32, [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _i32, _i32, C.c_float, _p]),
     "mtj_embed": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i32, _p, _p]),
     "mtj_layernorm": (_i32, [_p, _p, _p, _i64, _i64, _p, _i32, _p]),
     "mtj_xent": (_i32, [_p, _i64, _p, _i64, _i64, _p, _p, _p]),
-    "mtj_gemm": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, C.POINTER(InProj), _p]),
+    "mtj_gemm": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, C.POINTER(InProj), C.c_float, _p]),
     "mtj_gemm_splitk_work_bytes": (_i64, [_i64, _i64, _i64, _i32]),
-    "mtj_gemm_splitk": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, _p, _i64, _p]),
-    "mtj_gemm_splitk_ln": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _p, _i64, _p, _i64, _p, _p, _p, _i64, _i32, _p]),
-    "mtj_gemv": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p, _i32, C.POINTER(InProj), _p]),
+    "mtj_gemm_splitk": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, _p, _i64, C.c_float, _p]),
+    "mtj_gemm_splitk_ln": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _p, _i64, _p, _i64, _p, _p, _p, _i64, _i32,
+                                 C.c_float, _p]),
+    "mtj_gemv": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p, _i32, C.POINTER(InProj), C.POINTER(AttnMerge), _p]),
     "mtj_attn_prefill": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64, _i32, _p, _p]),
+    "mtj_attn_decode_splits": (_i32, [_i64, _i64, _i64]),
     "mtj_attn_decode_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),
+    "mtj_attn_decode_partials": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p, C.POINTER(AttnMerge), _p]),
     "mtj_attn_decode": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _i32, _i32, _p, _p]),
     "mtj_attn_decode_static_max_bytes": (_i64, []),
     "mtj_attn_decode_static": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _i32, _i32, _p]),
@@ -109,7 +118,9 @@ def dtype_code(torch_dtype) -> int:
         return F32
     if torch_dtype == torch.bfloat16:
         return BF16
-    raise ValueError(f"unsupported dtype {torch_dtype}: weights must be float32 or bfloat16")
+    if torch_dtype == torch.float16:
+        return F16
+    raise ValueError(f"unsupported dtype {torch_dtype}: float32, bfloat16 or float16")
 
 
 def stream_handle():

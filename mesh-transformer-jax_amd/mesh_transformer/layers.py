@@ -82,7 +82,8 @@ class EmbeddingShard:
 class TransformerLayerShard:
     """layers.py:229-366.  Returns the residual DELTA, like the reference; the caller adds x.
 
-    Decode state: {"k", "v": [1, H, Tcap, dh] device tensors in the weight dtype (k stored rotated,
+    Decode state: {"k", "v": [1, H, Tcap, dh] device tensors (float32 for a float32 model, float16 for a bfloat16 one;
+    k stored rotated,
     slot = position % Tcap), "tokens_decoded": int}.  decode_once updates k and v IN PLACE (the reference
     returns new arrays); the returned dict aliases the same tensors."""
 
@@ -158,8 +159,8 @@ class ProjectionShard:
         out = torch.empty(M, w.V, dtype=torch.float32, device=eng.device)
         with torch.cuda.device(eng.device):
             s = _abi.stream_handle()
-            h = torch.empty(M, w.d, dtype=w.torch_dtype, device=eng.device)
-            check(L.mtj_layernorm(ptr(x), ptr(w.pln_s), ptr(w.pln_o), M, w.d, ptr(h), w.dtype, s))
-            check(L.mtj_gemm(ptr(h), w.d, ptr(w.w_p), ptr(w.b_p), M, w.V, w.d, w.dtype, EPI_STORE, ptr(out), w.V, F32,
-                             None, s))
+            h = torch.empty(M, w.d, dtype=w.act_torch_dtype, device=eng.device)
+            check(L.mtj_layernorm(ptr(x), ptr(w.pln_s), ptr(w.pln_o), M, w.d, ptr(h), w.act_dtype, s))
+            check(L.mtj_gemm(ptr(h), w.d, ptr(w.w_p_mm), ptr(w.b_p), M, w.V, w.d, w.mm_dtype, EPI_STORE, ptr(out), w.V, F32,
+                             None, w.alpha_p, s))
         return out

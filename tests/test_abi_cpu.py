@@ -44,7 +44,10 @@ def test_struct_layouts_match_the_header():
     names = re.findall(r"\b([a-zA-Z_0-9]+)\s*(?:,|;)", re.sub(r"/\*.*?\*/", "", body, flags=re.S))
     assert names == [f[0] for f in _abi.InProj._fields_]
     assert ctypes.sizeof(_abi.InProj) % 8 == 0
-    body = text[text.index("typedef struct {", text.index("mtj_inproj;")):text.index("} mtj_next_embed;")]
+    body = text[text.index("typedef struct {", text.index("mtj_inproj;")):text.index("} mtj_attn_merge;")]
+    names = re.findall(r"\b([a-zA-Z_0-9]+)\s*(?:,|;)", re.sub(r"/\*.*?\*/", "", body, flags=re.S))
+    assert names == [f[0] for f in _abi.AttnMerge._fields_]
+    body = text[text.index("typedef struct {", text.index("mtj_attn_merge;")):text.index("} mtj_next_embed;")]
     names = re.findall(r"\b([a-zA-Z_0-9]+)\s*(?:,|;)", re.sub(r"/\*.*?\*/", "", body, flags=re.S))
     assert names == [f[0] for f in _abi.NextEmbed._fields_]
 
@@ -56,8 +59,11 @@ def test_argument_validation_needs_no_device():
     assert lib.mtj_layernorm(None, None, None, 1, 8, None, 0, None) == -1
     assert b"null pointer" in lib.mtj_last_error()
     with pytest.raises(ValueError):
-        _abi.check(lib.mtj_gemv(None, None, None, None, None, 8, 8, 0, 0, None, 0, None, None))
-    assert lib.mtj_attn_decode_work_bytes(1, 16, 256, 2047) == 16 * 32 * 258 * 4
+        _abi.check(lib.mtj_gemv(None, None, None, None, None, 8, 8, 0, 0, None, 0, None, None, None))
+    # one sequence of 16 heads: 8 key ranges per head (128 workgroups); 32 sequences fill the chip with one range each
+    assert lib.mtj_attn_decode_splits(1, 16, 2047) == 8 and lib.mtj_attn_decode_splits(32, 16, 2047) == 1
+    assert lib.mtj_attn_decode_splits(1, 16, 20) == 2          # never fewer than 16 slots per range at a full window
+    assert lib.mtj_attn_decode_work_bytes(1, 16, 256, 2047) == 16 * 8 * 260 * 4
     assert lib.mtj_sample_work_bytes(32, 50400) > 2 * 32 * 50400 * 8
 
 
@@ -89,3 +95,18 @@ def test_util_casts():
     b = to_bf16(t)
     assert b["a"]["w"].dtype == torch.bfloat16 and b["a"]["i"].dtype == torch.int32
     assert to_f32(b)["a"]["w"].dtype == torch.float32
+
+
+def test_session_workspace_covers_every_prompt_length():
+    """The out projection of a prefill is cut into MORE K ranges the FEWER rows it has, so the workspace of a session
+    sized for its longest prompt must also hold the partials of every shorter one (host-side sizes only)."""
+    from mesh_transformer import _abi
+    from mesh_transformer.engine import splitk_work_bound
+    lib = _abi.lib()
+    for dtype in (_abi.F32, _abi.F16, _abi.BF16):
+        for M_max, N, K in ((8 * 599, 4096, 20480), (700, 512, 2560), (2047, 4096, 20480), (100, 4096, 20480)):
+            bound = splitk_work_bound(M_max, N, K, dtype)
+            need = max(lib.mtj_gemm_splitk_work_bytes(m, N, K, dtype) for m in range(1, M_max + 1))
+            assert bound == need, (dtype, M_max, N, K)
+    # the case that used to fail: a session first sized for 8 x 599 rows, later used with 8 x 99
+    assert lib.mtj_gemm_splitk_work_bytes(8 * 99, 4096, 20480, _abi.F16) > lib.mtj_gemm_splitk_work_bytes(8 * 599, 4096, 20480, _abi.F16)

@@ -41,9 +41,11 @@ def max_err(got, ref):
     return float((got.double().cpu() - ref.double().cpu()).abs().max())
 
 
-TD = {"f32": torch.float32, "bf16": torch.bfloat16}
-# float32 path: the 1e-4 relative budget of the whole layer leaves ~1e-5 per kernel
-TOL = {"f32": 2e-6, "bf16": 6e-3}
+TD = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+# float32 path: the 1e-4 relative budget of the whole layer leaves ~1e-5 per kernel; 16-bit outputs carry their
+# own rounding (2^-9 relative for bfloat16, 2^-12 for float16)
+TOL = {"f32": 2e-6, "bf16": 6e-3, "f16": 8e-4}
+DTS = ["f32", "bf16", "f16"]
 
 
 # ------------------------------------------------------------------ pack / embed / layernorm
@@ -117,7 +119,7 @@ def _packed(w_haiku):
     return dst
 
 
-@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (32, 256, 128), (33, 300, 192), (128, 128, 512), (200, 1000, 256),
                                    (64, 520, 2560), (257, 96, 64)])
 def test_gemm_store_and_resid(L, dt, M, N, K):
@@ -130,25 +132,59 @@ def test_gemm_store_and_resid(L, dt, M, N, K):
     ref = A.double() @ Wh.double() + bias.double()
     out = torch.empty(M, N, device=DEV)
     a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, a.dtype_code(TD[dt]), a.EPI_STORE, a.ptr(out), N, 0,
-                       None, S()))
+                       None, 1.0, S()))
     torch.cuda.synchronize()
     assert rel_err(out, ref) < 5e-6, (dt, M, N, K)      # inputs are already rounded: only fp32 accumulation differs
     # RESID: x += A W + b, with a padded leading dimension
     x0 = torch.randn(M, N + 8, generator=g).to(DEV)
     x = x0.clone()
     a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, a.dtype_code(TD[dt]), a.EPI_RESID, a.ptr(x), N + 8, 0,
-                       None, S()))
+                       None, 1.0, S()))
     torch.cuda.synchronize()
     assert rel_err(x[:, :N], x0[:, :N].double() + ref) < 5e-6
     assert torch.equal(x[:, N:], x0[:, N:])
-    # bf16 output
-    ob = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
-    a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), None, M, N, K, a.dtype_code(TD[dt]), a.EPI_STORE, a.ptr(ob), N, 1, None, S()))
+    # 16-bit outputs
+    for odt in ("bf16", "f16"):
+        ob = torch.empty(M, N, dtype=TD[odt], device=DEV)
+        a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), None, M, N, K, a.dtype_code(TD[dt]), a.EPI_STORE, a.ptr(ob), N,
+                           a.dtype_code(TD[odt]), None, 1.0, S()))
+        torch.cuda.synchronize()
+        assert rel_err(ob, A.double() @ Wh.double()) < TOL[odt] / 2
+
+
+def test_pack_cvt_holds_bf16_weights_exactly_in_float16_and_alpha_undoes_the_scale(L):
+    """The matrix-core path of a bfloat16 model: weights go to float16 times a power of two (exact for every weight
+    whose scaled magnitude is a normal float16), the GEMM multiplies the accumulator by the inverse."""
+    a = abi()
+    g = torch.Generator().manual_seed(11)
+    M, N, K = 96, 384, 256
+    Wh = (torch.randn(K, N, generator=g) * 0.02).to(torch.bfloat16)
+    Wh[0, 0], Wh[1, 1], Wh[2, 2] = 0.11, -3e-6, 2e-9                 # the largest weight and two tiny ones
+    Wh = Wh.to(DEV)
+    scale = 2.0 ** 17                                                # 0.11 * 2^17 < 2^15
+    W16 = torch.empty(N, K, dtype=torch.float16, device=DEV)
+    a.check(L.mtj_pack_weight_cvt(a.ptr(Wh), N, K, N, a.ptr(W16), K, 0, 0, a.BF16, a.F16, scale, S()))
     torch.cuda.synchronize()
-    assert rel_err(ob, A.double() @ Wh.double()) < 3e-3
+    back = W16.double().T / scale
+    exact = Wh.double()
+    assert torch.equal(back[exact.abs() * scale >= 2.0 ** -14], exact[exact.abs() * scale >= 2.0 ** -14])
+    assert float((back - exact).abs().max()) <= 2.0 ** -25 / scale + 1e-300      # subnormal tail: half a step of 2^-24
+    A = torch.randn(M, K, generator=g).to(torch.float16).to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    out = torch.empty(M, N, device=DEV)
+    a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W16), a.ptr(bias), M, N, K, a.F16, a.EPI_STORE, a.ptr(out), N, 0, None,
+                       1.0 / scale, S()))
+    torch.cuda.synchronize()
+    assert rel_err(out, A.double() @ exact + bias.double()) < 5e-6
+    # saturation instead of infinity
+    big = torch.full((64, 64), 3.0e38, dtype=torch.bfloat16, device=DEV)
+    o16 = torch.empty(64, 64, dtype=torch.float16, device=DEV)
+    a.check(L.mtj_pack_weight_cvt(a.ptr(big), 64, 64, 64, a.ptr(o16), 64, 0, 0, a.BF16, a.F16, 1.0, S()))
+    torch.cuda.synchronize()
+    assert float(o16.float().max()) == 65504.0
 
 
-@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("M,N,K", [(32, 4096, 20480), (5, 512, 2560), (64, 260, 1024), (8, 50400, 4096), (3, 64, 64),
                                    (511, 4096, 20480), (200, 512, 2560), (700, 1024, 4096), (130, 4096, 20480), (300, 2048, 8192)])
 def test_gemm_splitk_matches_reference_and_is_deterministic(L, dt, M, N, K):
@@ -169,7 +205,7 @@ def test_gemm_splitk_matches_reference_and_is_deterministic(L, dt, M, N, K):
     for _ in range(2):
         out = torch.empty(M, N, device=DEV)
         a.check(L.mtj_gemm_splitk(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_STORE, a.ptr(out), N, 0,
-                                  a.ptr(work), work.numel(), S()))
+                                  a.ptr(work), work.numel(), 1.0, S()))
         torch.cuda.synchronize()
         outs.append(out)
     assert rel_err(outs[0], ref) < 5e-6
@@ -177,16 +213,16 @@ def test_gemm_splitk_matches_reference_and_is_deterministic(L, dt, M, N, K):
     x0 = torch.randn(M, N, generator=g).to(DEV)
     x = x0.clone()
     a.check(L.mtj_gemm_splitk(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_RESID, a.ptr(x), N, 0,
-                              a.ptr(work), work.numel(), S()))
+                              a.ptr(work), work.numel(), 1.0, S()))
     torch.cuda.synchronize()
     assert rel_err(x, x0.double() + ref) < 5e-6
     if nb:
         with pytest.raises(ValueError):                  # a work buffer that is too small is refused
             a.check(L.mtj_gemm_splitk(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_STORE, a.ptr(out), N, 0,
-                                      a.ptr(work), nb - 4, S()))
+                                      a.ptr(work), nb - 4, 1.0, S()))
 
 
-@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("M,N,K", [(32, 4096, 20480), (5, 512, 2560), (3, 64, 64), (8, 1024, 4096)])
 def test_gemm_splitk_with_the_following_layernorm(L, dt, M, N, K):
     """The residual reduce that also normalises the rows it completes: x as from mtj_gemm_splitk (bit for bit), h as
@@ -205,29 +241,29 @@ def test_gemm_splitk_with_the_following_layernorm(L, dt, M, N, K):
     x0 = torch.randn(M, N, generator=g).to(DEV)
     x_ref = x0.clone()
     a.check(L.mtj_gemm_splitk(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_RESID, a.ptr(x_ref), N, 0,
-                              a.ptr(work), work.numel(), S()))
-    for h_dt in ("f32", "bf16"):
+                              a.ptr(work), work.numel(), 1.0, S()))
+    for h_dt in DTS:
         x = x0.clone()
         h = torch.zeros(M, N, dtype=TD[h_dt], device=DEV)
         a.check(L.mtj_gemm_splitk_ln(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.ptr(x), N, a.ptr(work),
-                                     work.numel(), a.ptr(sc), a.ptr(of), a.ptr(h), N, a.dtype_code(TD[h_dt]), S()))
+                                     work.numel(), a.ptr(sc), a.ptr(of), a.ptr(h), N, a.dtype_code(TD[h_dt]), 1.0, S()))
         torch.cuda.synchronize()
         assert torch.equal(x, x_ref)
         ref = O.replicated_layer_norm(x.double().cpu(), sc.double().cpu(), of.double().cpu()).to(DEV)
-        assert rel_err(h, ref) < (6e-6 if h_dt == "f32" else 4e-3)
+        assert rel_err(h, ref) < {"f32": 6e-6, "bf16": 4e-3, "f16": 5e-4}[h_dt]
 
 
 def test_gemm_rejects_bad_arguments(L):
     a = abi()
     A = torch.zeros(4, 48, device=DEV)
     with pytest.raises(ValueError):   # K not a multiple of the k-tile
-        a.check(L.mtj_gemm(a.ptr(A), 48, a.ptr(A), None, 4, 4, 48, 0, a.EPI_STORE, a.ptr(A), 4, 0, None, S()))
+        a.check(L.mtj_gemm(a.ptr(A), 48, a.ptr(A), None, 4, 4, 48, 0, a.EPI_STORE, a.ptr(A), 4, 0, None, 1.0, S()))
     with pytest.raises(ValueError):   # INPROJ without geometry
-        a.check(L.mtj_gemm(a.ptr(A), 32, a.ptr(A), None, 4, 4, 32, 0, a.EPI_INPROJ, None, 0, 0, None, S()))
+        a.check(L.mtj_gemm(a.ptr(A), 32, a.ptr(A), None, 4, 4, 32, 0, a.EPI_INPROJ, None, 0, 0, None, 1.0, S()))
 
 
 # ------------------------------------------------------------------ GEMV
-@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("N,K", [(512, 256), (28672, 4096), (4096, 20480), (50400, 4096), (514, 2560), (6, 520),
                                  # whole-tile rows with 0 or 1, exactly 1, 3, and 4-or-5 tiles per wavefront
                                  (8, 4096), (4096, 4096), (12288, 4096), (9000, 8192)])
@@ -241,13 +277,13 @@ def test_gemv_store_resid_and_layernorm(L, dt, N, K):
     ref = x.double() @ Wh.double() + bias.double()
     out = torch.empty(N, device=DEV)
     a.check(L.mtj_gemv(a.ptr(x), None, None, a.ptr(W), a.ptr(bias), N, K, a.dtype_code(TD[dt]), a.EPI_STORE, a.ptr(out), 0,
-                       None, S()))
+                       None, None, S()))
     torch.cuda.synchronize()
     assert rel_err(out, ref) < 5e-6
     y0 = torch.randn(N, generator=g).to(DEV)
     y = y0.clone()
     a.check(L.mtj_gemv(a.ptr(x), None, None, a.ptr(W), a.ptr(bias), N, K, a.dtype_code(TD[dt]), a.EPI_RESID, a.ptr(y), 0,
-                       None, S()))
+                       None, None, S()))
     torch.cuda.synchronize()
     assert rel_err(y, y0.double() + ref) < 5e-6
     if K <= 16384:
@@ -255,7 +291,7 @@ def test_gemv_store_resid_and_layernorm(L, dt, N, K):
         of = (0.1 * torch.randn(K, generator=g)).to(DEV)
         xr = (x * 2 + 0.7)
         a.check(L.mtj_gemv(a.ptr(xr), a.ptr(sc), a.ptr(of), a.ptr(W), a.ptr(bias), N, K, a.dtype_code(TD[dt]), a.EPI_STORE,
-                           a.ptr(out), 0, None, S()))
+                           a.ptr(out), 0, None, None, S()))
         torch.cuda.synchronize()
         h = O.replicated_layer_norm(xr.double().cpu()[None], sc.double().cpu(), of.double().cpu())[0].to(DEV)
         assert rel_err(out, h @ Wh.double() + bias.double()) < 6e-6
@@ -285,33 +321,28 @@ def _inproj_reference(cfg, p, x64, positions):
     return rot(q), rot(k), v, O.gelu_tanh(h @ l.w1 + l.b1), h
 
 
-@pytest.mark.parametrize("dt", ["f32", "bf16"])
-@pytest.mark.parametrize("shape", ["tiny", "head256"])
-def test_inproj_gemm_prefill_with_left_padding(dt, shape):
+def _run_inproj_prefill(cfg, p, dt, B, Tp, Tcap, pads, seed):
+    """LayerNorm + fused q|v|k|fc_in GEMM of layer 0 through the engine's buffers; compares q, the K/V window, V^T and
+    gelu(fc_in) of every real row with the float64 oracle.  A bfloat16 model runs its matrix-core path in float16."""
     from mesh_transformer.engine import Engine
     a = abi()
-    cfg = dict(layers=1, d_model=512, n_heads=8, n_vocab=64, pe="rotary", pe_rotary_dims=32, cores_per_replica=1) \
-        if shape == "tiny" else \
-        dict(layers=1, d_model=512, n_heads=2, n_vocab=64, pe="rotary", pe_rotary_dims=64, cores_per_replica=1)
-    p = _layer_params(cfg, 3, dt)
+    d = cfg["d_model"]
     eng = Engine(cfg, {k: {n: v.to(DEV) for n, v in m.items()} for k, m in p.items()}, DEV, layer_ids=[0], embed=False, proj=False)
-    B, Tp, Tcap = 2, 40, 50
-    pads = [0, 7]
-    ses = eng.session(B, Tcap, Tp, 64)
-    g = torch.Generator().manual_seed(4)
-    x = torch.randn(B * Tp, 512, generator=g).to(DEV)
+    ses = eng.session(B, Tcap, Tp, Tp + 8)
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B * Tp, d, generator=g).to(DEV)
     pos0 = torch.tensor([-pd for pd in pads], dtype=torch.int32, device=DEV)
     w = eng.w
     L = a.lib()
     h = ses.h_pf[:B * Tp]
     act = ses.act_pf[:B * Tp]
-    a.check(L.mtj_layernorm(a.ptr(x), a.ptr(w.ln_s[0]), a.ptr(w.ln_o[0]), B * Tp, 512, a.ptr(h), w.dtype, S()))
-    ip = eng._inproj(ses, 0, Tp, pos0, ses.q_pf, w.dtype, act, w.dtype, ses.vt)
-    a.check(L.mtj_gemm(a.ptr(h), 512, a.ptr(w.w_in[0]), a.ptr(w.b1[0]), B * Tp, 3 * 512 + 2048, 512, w.dtype, a.EPI_INPROJ,
-                       None, 0, 0, C.byref(ip), S()))
+    a.check(L.mtj_layernorm(a.ptr(x), a.ptr(w.ln_s[0]), a.ptr(w.ln_o[0]), B * Tp, d, a.ptr(h), w.act_dtype, S()))
+    ip = eng._inproj(ses, 0, Tp, pos0, ses.q_pf, w.act_dtype, act, w.act_dtype, ses.vt)
+    a.check(L.mtj_gemm(a.ptr(h), d, a.ptr(w.w_in_mm[0]), a.ptr(w.b1[0]), B * Tp, 3 * d + 4 * d, d, w.mm_dtype, a.EPI_INPROJ,
+                       None, 0, 0, C.byref(ip), w.alpha_in[0], S()))
     torch.cuda.synchronize()
     H, dh = eng.H, eng.dh
-    tol = TOL[dt] * (3 if dt == "f32" else 1.5)
+    tol = 6e-6 if dt == "f32" else 1.2e-3        # float16 operand and float16 storage: 2^-12 relative each
     for b in range(B):
         pd = pads[b]
         rows = x[b * Tp + pd:(b + 1) * Tp].double().cpu()
@@ -324,9 +355,48 @@ def test_inproj_gemm_prefill_with_left_padding(dt, shape):
         assert rel_err(kk, k_ref) < tol and rel_err(vv, v_ref) < tol
         vt = ses.vt.reshape(B, H, dh, ses.ldvt)[b, :, :, :Tp - pd].permute(2, 0, 1)
         assert torch.equal(vt.contiguous(), vv.contiguous())
-        assert rel_err(act[b * Tp + pd:(b + 1) * Tp, 512:], g_ref) < tol
+        assert rel_err(act[b * Tp + pd:(b + 1) * Tp, d:], g_ref) < tol
         # nothing was written for padding rows: the slots after the real tokens are still zero
         assert float(ses.kc[0][b, :, Tp - pd:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("shape", ["tiny", "head256"])
+def test_inproj_gemm_prefill_with_left_padding(dt, shape):
+    cfg = dict(layers=1, d_model=512, n_heads=8, n_vocab=64, pe="rotary", pe_rotary_dims=32, cores_per_replica=1) \
+        if shape == "tiny" else \
+        dict(layers=1, d_model=512, n_heads=2, n_vocab=64, pe="rotary", pe_rotary_dims=64, cores_per_replica=1)
+    _run_inproj_prefill(cfg, _layer_params(cfg, 3, dt), dt, B=2, Tp=40, Tcap=50, pads=[0, 7], seed=4)
+
+
+def test_inproj_gemm_on_the_256x256_direct_to_lds_kernel():
+    """M = 1024 rows x N = 14336 columns is 4 x 56 = 224 tiles of 256 x 256: mtj_gemm dispatches gemm_dma_kernel (at
+    least 200 such tiles), whose 8-wavefront epilogue (RoPE, K/V ring, V^T, GELU) the small shapes never reach."""
+    cfg = dict(layers=1, d_model=2048, n_heads=8, n_vocab=64, pe="rotary", pe_rotary_dims=64, cores_per_replica=1)
+    _run_inproj_prefill(cfg, _layer_params(cfg, 9, "bf16"), "bf16", B=2, Tp=512, Tcap=600, pads=[0, 37], seed=10)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_gemm_resid_and_store_on_the_256x256_direct_to_lds_kernel(L, dt):
+    """M = N = 4096 is 256 tiles of 256 x 256, so mtj_gemm itself (no K split) runs gemm_dma_kernel with the RESID and
+    STORE epilogues; K = 4096 * 5 is the out|fc_out depth of the 6B model.  Reference: float64 product on the GPU."""
+    a = abi()
+    g = torch.Generator().manual_seed(21)
+    M, N, K = 4096, 4096, 20480
+    A = torch.randn(M, K, generator=g).to(TD[dt]).to(DEV)
+    Wh = (torch.randn(K, N, generator=g) * 0.02).to(TD[dt]).to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    W = _packed(Wh)
+    ref = A.double() @ Wh.double() + bias.double()
+    x0 = torch.randn(M, N, generator=g).to(DEV)
+    x = x0.clone()
+    code = a.dtype_code(TD[dt])
+    a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_RESID, a.ptr(x), N, 0, None, 1.0, S()))
+    out = torch.empty(M - 100, N, device=DEV)                 # a ragged last row tile
+    a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), a.ptr(bias), M - 100, N, K, code, a.EPI_STORE, a.ptr(out), N, 0, None, 0.5, S()))
+    torch.cuda.synchronize()
+    assert rel_err(x, x0.double() + ref) < 5e-6
+    assert rel_err(out, 0.5 * (ref[:M - 100] - bias.double()) + bias.double()) < 5e-6
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
@@ -345,10 +415,10 @@ def test_inproj_gemv_decode_appends_to_ring(dt):
         ses.pos.fill_(pos)
         ip = eng._inproj(ses, 0, 1, ses.pos, ses.q, 0, ses.act, 0, None)
         a.check(L.mtj_gemv(a.ptr(x), a.ptr(w.ln_s[0]), a.ptr(w.ln_o[0]), a.ptr(w.w_in[0]), a.ptr(w.b1[0]), 3 * 512 + 2048, 512,
-                           w.dtype, a.EPI_INPROJ, None, 0, C.byref(ip), S()))
+                           w.dtype, a.EPI_INPROJ, None, 0, C.byref(ip), None, S()))
         torch.cuda.synchronize()
         q_ref, k_ref, v_ref, g_ref, _ = _inproj_reference(cfg, p, x.double().cpu(), np.array([pos]))
-        tol = TOL[dt] * 3 if dt == "f32" else 5e-3
+        tol = TOL[dt] * 3 if dt == "f32" else 5e-4       # the K/V window of a bfloat16 model is float16
         assert rel_err(ses.q.reshape(1, eng.H, eng.dh), q_ref) < 3e-6
         assert rel_err(ses.kc[0][0, :, pos % Tcap][None], k_ref) < tol
         assert rel_err(ses.vc[0][0, :, pos % Tcap][None], v_ref) < tol
@@ -366,7 +436,10 @@ def _attn_reference(q, k, v, n_pad):
     return torch.einsum("htT,Thd->thd", w, v).reshape(T, H * dh)[n_pad:]
 
 
-@pytest.mark.parametrize("dt", ["f32", "bf16"])
+ATT_TOL = {"f32": 3e-6, "bf16": 8e-3, "f16": 1e-3}      # probabilities and the output are rounded to the storage type
+
+
+@pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("dh,H", [(64, 3), (256, 2)])
 @pytest.mark.parametrize("Tp", [1, 33, 128, 200])
 def test_attn_prefill(L, dt, dh, H, Tp):
@@ -395,7 +468,7 @@ def test_attn_prefill(L, dt, dh, H, Tp):
         ref = _attn_reference(q[b].permute(1, 0, 2).double().cpu(), kk[b].permute(1, 0, 2).double().cpu(),
                               vv[b].permute(1, 0, 2).double().cpu(), pd)
         got = out[b * Tp + pd:(b + 1) * Tp, :H * dh]
-        assert rel_err(got, ref) < (3e-6 if dt == "f32" else 8e-3), (dt, dh, Tp, b)
+        assert rel_err(got, ref) < ATT_TOL[dt], (dt, dh, Tp, b)
         assert float(out[b * Tp:b * Tp + pd, :H * dh].float().abs().max() if pd else 0.0) == 0.0   # padding rows: zeros
     assert torch.all(out[:, H * dh:] == 7.0)
     # evaluation mask (transformer_shard.py:130): keys beyond key_limit[b] are hidden from every query
@@ -417,12 +490,46 @@ def test_attn_prefill(L, dt, dh, H, Tp):
             bias = O.MASK * (1.0 - torch.tril(torch.ones(Tp, Tp, dtype=torch.float64)))
             bias = bias + (torch.arange(Tp) > lim[b]).double() * -1e10
             ref = torch.einsum("htT,Thd->thd", torch.softmax(sc + bias, -1), vq).reshape(Tp, H * dh)
-            assert rel_err(out[b * Tp:(b + 1) * Tp, :H * dh], ref) < (3e-6 if dt == "f32" else 8e-3), (dt, dh, Tp, b)
+            assert rel_err(out[b * Tp:(b + 1) * Tp, :H * dh], ref) < ATT_TOL[dt], (dt, dh, Tp, b)
 
 
-@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_attn_prefill_full_context_d256(L, dt):
+    """2048 queries per sequence at d_head 256 with ragged left padding: 16 query blocks per head, dispatched longest
+    first, every key tile count from 1 to 64 - the shape of the 6B prefill, against the float64 reference."""
+    a = abi()
+    g = torch.Generator().manual_seed(77)
+    B, H, Tp, dh = 2, 2, 2048, 256
+    Tcap, pads = Tp, [0, 301]
+    ldvt = Tp + 64
+    q = torch.randn(B, H, Tp, dh, generator=g).to(TD[dt]).to(DEV)
+    kk = torch.randn(B, H, Tp, dh, generator=g).to(TD[dt]).to(DEV)
+    vv = torch.randn(B, H, Tp, dh, generator=g).to(TD[dt]).to(DEV)
+    kc = torch.zeros(B, H, Tcap, dh, dtype=TD[dt], device=DEV)
+    vt = torch.full((B, H, dh, ldvt), float("nan"), dtype=TD[dt], device=DEV)
+    for b in range(B):
+        n = Tp - pads[b]
+        kc[b, :, :n] = kk[b, :, pads[b]:]
+        vt[b, :, :, :n] = vv[b, :, pads[b]:].permute(0, 2, 1)
+    pos0 = torch.tensor([-pd for pd in pads], dtype=torch.int32, device=DEV)
+    out = torch.zeros(B * Tp, H * dh, dtype=TD[dt], device=DEV)
+    a.check(L.mtj_attn_prefill(a.ptr(q), a.ptr(kc), a.ptr(vt), a.ptr(pos0), B, H, Tp, Tcap, dh, ldvt, a.ptr(out), H * dh,
+                               a.dtype_code(TD[dt]), None, S()))
+    torch.cuda.synchronize()
+    for b in range(B):
+        pd = pads[b]
+        ref = _attn_reference(q[b].permute(1, 0, 2).double().cpu(), kk[b].permute(1, 0, 2).double().cpu(),
+                              vv[b].permute(1, 0, 2).double().cpu(), pd)
+        got = out[b * Tp + pd:(b + 1) * Tp].double().cpu()
+        assert rel_err(got, ref) < ATT_TOL[dt], (dt, b)
+        # no row is far off either (a wrong tile or a stale buffer would show as a few bad rows)
+        row_err = (got - ref).norm(dim=1) / ref.norm(dim=1)
+        assert float(row_err.max()) < 4 * ATT_TOL[dt], (dt, b, int(row_err.argmax()))
+
+
+@pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("dh,H", [(64, 8), (256, 16)])
-@pytest.mark.parametrize("Tcap,positions", [(7, [0, 6, 9]), (300, [0, 150, 299]), (2047, [511, 2046, 5000]),
+@pytest.mark.parametrize("Tcap,positions", [(7, [0, 6, 9]), (300, [0, 150, 299]), (2047, [511, 2046, 5000]), (2047, [700]),
                                             # many sequences, ragged positions, some beyond the window
                                             (1000, [(i * 131) % 1300 for i in range(24)])])
 def test_attn_decode_window(L, dt, dh, H, Tcap, positions):
@@ -443,6 +550,43 @@ def test_attn_decode_window(L, dt, dh, H, Tcap, positions):
         s = torch.einsum("hd,hTd->hT", q[b].double(), kc[b, :, :n].double()) / math.sqrt(dh)
         ref = torch.einsum("hT,hTd->hd", torch.softmax(s, -1), vc[b, :, :n].double()).reshape(-1)
         assert rel_err(out[b, :H * dh], ref) < 3e-6, (dt, dh, Tcap, p)
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+@pytest.mark.parametrize("dh,H,F", [(64, 8, 2048), (256, 16, 16384)])
+@pytest.mark.parametrize("Tcap,p", [(2047, 650), (2047, 2046), (130, 3), (9, 40)])
+def test_attn_decode_partials_merged_by_the_out_projection_gemv(L, dt, dh, H, F, Tcap, p):
+    """Batch 1: the per-range partials of the one-token attention are merged by mtj_gemv while it stages its input;
+    x += [attention | gelu] @ W_out + b must equal the float64 evaluation of layers.py:275-285, 290, 313."""
+    a = abi()
+    g = torch.Generator().manual_seed(Tcap + dh + p)
+    d = H * dh
+    q = torch.randn(1, H, dh, generator=g).to(DEV)
+    kc = torch.randn(1, H, Tcap, dh, generator=g).to(TD[dt]).to(DEV)
+    vc = torch.randn(1, H, Tcap, dh, generator=g).to(TD[dt]).to(DEV)
+    pos = torch.tensor([p], dtype=torch.int32, device=DEV)
+    work = torch.zeros(L.mtj_attn_decode_work_bytes(1, H, dh, Tcap), dtype=torch.uint8, device=DEV)
+    am = a.AttnMerge()
+    a.check(L.mtj_attn_decode_partials(a.ptr(q), a.ptr(kc), a.ptr(vc), a.ptr(pos), 1, H, Tcap, dh, a.dtype_code(TD[dt]),
+                                       a.ptr(work), C.byref(am), S()))
+    assert am.splits == L.mtj_attn_decode_splits(1, H, Tcap) and am.n_heads == H and am.d_head == dh
+    wdt = "f32" if dt == "f32" else "bf16"
+    act = torch.randn(1, d + F, generator=g).to(DEV)
+    act[:, :d] = float("nan")                                   # the attention columns must come from the partials
+    Wh = (torch.randn(d + F, d, generator=g) * 0.02).to(TD[wdt]).to(DEV)
+    W = _packed(Wh)
+    bias = torch.randn(d, generator=g).to(DEV)
+    x0 = torch.randn(d, generator=g).to(DEV)
+    x = x0.clone()
+    a.check(L.mtj_gemv(a.ptr(act), None, None, a.ptr(W), a.ptr(bias), d, d + F, a.dtype_code(TD[wdt]), a.EPI_RESID, a.ptr(x),
+                       0, None, C.byref(am), S()))
+    torch.cuda.synchronize()
+    n = min(p + 1, Tcap)
+    sc = torch.einsum("hd,hTd->hT", q[0].double(), kc[0, :, :n].double()) / math.sqrt(dh)
+    att = torch.einsum("hT,hTd->hd", torch.softmax(sc, -1), vc[0, :, :n].double()).reshape(-1)
+    inp = torch.cat([att, act[0, d:].double()])
+    ref = x0.double() + inp @ Wh.double() + bias.double()
+    assert rel_err(x, ref) < 5e-6, (dt, dh, Tcap, p)
 
 
 # ------------------------------------------------------------------ samplers: bit-exact against the oracle

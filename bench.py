@@ -12,7 +12,11 @@ Also reported on the same line:
                 algorithmic bytes of one launch / its average duration (HIP events), against 8 TB/s
   step_hbm      whole-step algorithmic bytes / measured step time
   prefill       the 511-token prefill of the same run, and one full-shape layer at [8 x 2048] tokens
-                (BASELINE config 2), as TFLOP/s against the 2.5 PFLOP/s bf16 MFMA peak
+                (BASELINE config 2), as TFLOP/s against the 2.5 PFLOP/s 16-bit MFMA peak
+  decode_b32    BASELINE config 4 on a bounded run: batch 32, 1024-token prompts padded to 2048, nucleus sampling
+                (top_p 0.9, temperature 0.8, host Philox(3) uniforms), ms/step and algorithmic HBM fraction
+  forward_16x2048  BASELINE config 5: full-context forward of 16 x 2048 tokens with the 50400-wide logits at
+                every position, TFLOP/s against the MFMA peak
   cpu_baseline  the CPU oracle (torch float32 on the host cores) on a bounded sample of the workload
 """
 import argparse
@@ -127,6 +131,58 @@ def time_prefill_layer(net, B=8, T=2048, reps=5):
     return a.elapsed_time(b) * 1e-3 / reps
 
 
+def time_decode_b32(net, cfg, B=32, P=1024, L=2048, warm=9, steps=64):
+    """BASELINE config 4, bounded: batch 32 nucleus decode after 1024-token prompts (the K/V window holds 1024 ..
+    1024 + warm + steps keys per sequence in the timed region; the full run would go on to 2047)."""
+    import numpy as np
+    from oracle import gptj_oracle as O
+    G = warm + steps
+    u = np.random.Generator(np.random.Philox(3)).random((B, G))
+    ctx = O.left_pad(O.seeded_prompt(3, B, P), L)
+    opts = {"top_p": np.full(B, 0.9), "temp": np.full(B, 0.8)}
+    tm = {"warmup": warm}
+    net.generate(ctx, np.full(B, P), G, opts, uniforms=u)             # untimed: allocates, records the graphs
+    net.generate(ctx, np.full(B, P), G, opts, uniforms=u, timing=tm)
+    ms = tm["decode_s"] * 1e3 / tm["decode_steps"]
+    ctx_mean = (P - 1) + warm + (steps - 1) / 2.0
+    nbytes = decode_bytes_per_step(cfg, ctx_mean, B)
+    net.engine().sessions.pop((B, L - 1), None)
+    return {"ms_per_step": ms, "tok_s": B * 1e3 / ms, "batch": B, "prompt": P, "steps": steps, "ctx_mean": ctx_mean,
+            "sampler": "nucleus top_p 0.9 temp 0.8, host Philox(3) uniforms",
+            "prefill_ms": tm["prefill_s"] * 1e3, "prefill_tok_s": tm["prefill_tokens"] / tm["prefill_s"],
+            "step_hbm": {"bytes": nbytes, "achieved": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s",
+                         "frac": nbytes / (ms * 1e-3) / HBM_PEAK}}
+
+
+def time_forward_16x2048(net, cfg, B=16, L=2048):
+    """BASELINE config 5: every-position logits of B x L uniform-random tokens (seed 4)."""
+    import numpy as np
+    import torch
+    rng = np.random.Generator(np.random.Philox(4))
+    ctx = rng.integers(0, 50257, (B, L)).astype(np.uint32)
+    net.forward(ctx)                                                   # untimed: allocates
+    tm = {}
+    out = net.forward(ctx, timing=tm)
+    del out
+    net.engine().sessions.pop((B, L), None)
+    torch.cuda.empty_cache()
+    d, F, n, V = cfg["d_model"], 4 * cfg["d_model"], cfg["layers"], cfg["n_vocab"]
+    fl = B * L * 2 * (n * (4 * d * d + 2 * d * F) + d * V) + B * n * 4 * d * L * (L + 1) / 2
+    t = tm["forward_s"]
+    return {"ms": t * 1e3, "tok_s": B * L / t, "tflops": fl / t / 1e12, "frac_mfma": fl / t / MFMA_BF16_PEAK,
+            "flops": "dense 2*params per token + causal attention 4*d*(t+1) per query"}
+
+
+def cpu_model_name():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(net, cfg, n_layers=4, steps=8, prompt=512, L=2048):
     """The CPU oracle (torch float32, all host threads) on a bounded sample: the first `n_layers` layers of the
     same weights at full shape plus embedding and logits projection; 512-token prompt left-padded to 2048,
@@ -161,7 +217,7 @@ def cpu_baseline(net, cfg, n_layers=4, steps=8, prompt=512, L=2048):
     t_step = float(np.median(per))
     t_full = (t_step - t_proj) * cfg["layers"] / n_layers + t_proj
     return {
-        "value": 1.0 / t_full, "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
+        "value": 1.0 / t_full, "unit": "tok/s", "cores": torch.get_num_threads(), "cpu": cpu_model_name(), "kind": "port",
         "sample": f"CPU oracle (torch float32), {n_layers} of {cfg['layers']} layers at full shape + logits, "
                   f"{prompt}-token prompt padded to {L}, {steps} decode steps (median {t_step * 1e3:.1f} ms/step for "
                   f"{n_layers} layers, prefill {t1 - t0:.1f} s); per-step time extrapolated linearly to {cfg['layers']} layers",
@@ -282,7 +338,12 @@ def main():
         "roofline": roofline,
         "step_hbm": {"bytes": step_bytes, "achieved": step_bw / 1e9, "unit": "GB/s", "frac": step_bw / HBM_PEAK},
         "prefill": prefill,
+        "precision": "bf16 weights; batch-1 decode multiplies them with float32 activations, the matrix-core paths "
+                     "(prefill, batched decode) with float16 activations and float16 copies of the same weight values",
     }
+    if not args.no_extras:
+        res["decode_b32"] = time_decode_b32(net, cfg)
+        res["forward_16x2048"] = time_forward_16x2048(net, cfg)
     if not args.no_cpu:
         res["cpu_baseline"] = cpu_baseline(net, cfg)
     print(json.dumps(res))

@@ -156,33 +156,42 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // ---------------------------------------------------------------- merge of one-token attention partials
 // Partials of one (sequence, head): wb[s * (dh + MTJ_DEC_PAD)] = {max, sum, -, -, V[dh]} for key range s < S <= 8.
-// Returns elements e .. e+3 of sum_s exp(max_s - max) V_s / sum_s exp(max_s - max) sum_s.  Every load is issued
-// before the first is used and none depends on another; ranges beyond S read range S-1 again with weight 0.
+// Returns elements e .. e+3 of sum_s exp(max_s - max) V_s / sum_s exp(max_s - max) sum_s.  The ranges are taken four at
+// a time with a running maximum (four vectors and eight statistics in registers at once: the callers have their
+// weight tiles in registers too); inside a batch every load is issued before the first is used.  Ranges beyond S
+// read range S-1 again with weight 0.
 constexpr int MTJ_DEC_MAXS = 8;
 constexpr int MTJ_DEC_PAD = 4;
 __device__ __forceinline__ floatx4 mtj_merge_partials(const float* __restrict__ wb, int S, int dh, int e) {
-  float m[MTJ_DEC_MAXS], l[MTJ_DEC_MAXS];
-  floatx4 v[MTJ_DEC_MAXS];
-#pragma unroll
-  for (int s = 0; s < MTJ_DEC_MAXS; ++s) {
-    const float* p = wb + (int64_t)(s < S ? s : S - 1) * (dh + MTJ_DEC_PAD);
-    m[s] = p[0];
-    l[s] = p[1];
-    v[s] = *reinterpret_cast<const floatx4*>(p + MTJ_DEC_PAD + e);
-  }
-  float mm = -INFINITY;
-#pragma unroll
-  for (int s = 0; s < MTJ_DEC_MAXS; ++s) {
-    if (s >= S) m[s] = -INFINITY;
-    mm = fmaxf(mm, m[s]);
-  }
+  float mm = -INFINITY, lt = 0.f;
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-  float lt = 0.f;
+  for (int s0 = 0; s0 < S; s0 += 4) {
+    float m[4], l[4];
+    floatx4 v[4];
 #pragma unroll
-  for (int s = 0; s < MTJ_DEC_MAXS; ++s) {
-    const float f = (m[s] == -INFINITY) ? 0.f : __expf(m[s] - mm);    // an empty range has max -inf
-    lt = fmaf(f, l[s], lt);
-    acc += f * v[s];
+    for (int i = 0; i < 4; ++i) {
+      const float* p = wb + (int64_t)(s0 + i < S ? s0 + i : S - 1) * (dh + MTJ_DEC_PAD);
+      m[i] = p[0];
+      l[i] = p[1];
+      v[i] = *reinterpret_cast<const floatx4*>(p + MTJ_DEC_PAD + e);
+    }
+    float mb = mm;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (s0 + i >= S) m[i] = -INFINITY;
+      mb = fmaxf(mb, m[i]);
+    }
+    if (mb == -INFINITY) continue;                                      // only empty ranges so far
+    const float r = (mm == -INFINITY) ? 0.f : __expf(mm - mb);
+    lt *= r;
+    acc *= r;
+    mm = mb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float f = (m[i] == -INFINITY) ? 0.f : __expf(m[i] - mm);    // an empty range has max -inf
+      lt = fmaf(f, l[i], lt);
+      acc += f * v[i];
+    }
   }
   const float inv = lt > 0.f ? 1.0f / lt : 0.f;
   return acc * inv;

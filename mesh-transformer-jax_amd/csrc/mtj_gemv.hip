@@ -73,7 +73,9 @@ struct gemv_args {
 // contiguous run of whole tiles, which is streamed with two tiles in flight - the next one is requested before the
 // current one is consumed, so a wavefront never has an empty memory queue - and no load is conditional.  (Dealing
 // the rows out round-robin instead, so that the chip reads one contiguous window at a time, streams ~5 % faster in
-// a plain read but scatters every lane's epilogue loads and stores: 43.5 us against 40.2 for the 235 MB launch.)
+// a plain read but not here: 43.5 us against 40.2 for the 235 MB launch with every lane's epilogue scattered, 40.9
+// against 39.4 with the row sums routed through LDS so that one thread finishes a row and adjacent threads adjacent
+// rows; cutting the rows into 1 KiB pieces so that consecutive wavefronts read consecutive KiB takes 49.7 us.)
 // MERGE: the leading inputs are merged from one-token attention partials (a.am) instead of being read from x.
 template <typename T, int U, bool FULL, bool MERGE>
 __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {

@@ -2,19 +2,41 @@
 (ReplicatedLayerNorm, EmbeddingShard, TransformerLayerShard, ProjectionShard, rotary helpers), as thin
 wrappers over the HIP kernels so that every seam of the model can be compared on its own.
 
-The reference modules are haiku modules that pull their parameters from the enclosing transform; here
-each module is given the parameter tree explicitly (`params`, haiku names, leading shard axis of 1).
+The reference modules are haiku modules: their constructors take (config, name, ...) and the parameters come from
+the enclosing hk.transform.  The constructors here have the reference's positional arguments; the parameter tree
+(haiku names, leading shard axis of 1) comes from the enclosing `with layers.transform(tree):` block - the stand-in
+for hk.transform(...).apply(params, ...) - or from the keyword-only `params=` argument.
 Inputs and outputs are float32 CUDA tensors shaped like the reference's per-sequence arrays
 ([tokens, d_model]); attn_bias must be 0 (only pe == "rotary" is on this path).
+The kernels are reached through the torch.ops.mtj operators (mesh_transformer.ops) and the engine.
 """
-import ctypes as C
+import contextlib
 
 import numpy as np
 import torch
 
-from . import _abi
-from ._abi import EPI_STORE, F32, check, ptr
+from . import ops  # noqa: F401  (registers torch.ops.mtj.*)
 from .engine import ROOT, Engine, _f32, rotary_tables
+
+_AMBIENT = []
+
+
+@contextlib.contextmanager
+def transform(params):
+    """Parameter scope of the modules constructed inside it (what hk.transform(...).apply(params, ...) provides)."""
+    _AMBIENT.append(params)
+    try:
+        yield params
+    finally:
+        _AMBIENT.pop()
+
+
+def _tree(params):
+    if params is not None:
+        return params
+    if _AMBIENT:
+        return _AMBIENT[-1]
+    raise RuntimeError("no parameters in scope: construct the module inside `with layers.transform(tree):` or pass params=")
 
 
 def fixed_pos_embedding(x, seq_dim=0):
@@ -36,47 +58,38 @@ def _f32_in(x, dev):
 
 
 class ReplicatedLayerNorm:
-    """layers.py:12-36."""
+    """layers.py:12-36: ReplicatedLayerNorm(offset=True).  Its parameters {"scale", "offset"} ([1, d] each) are the
+    module `name` of the tree in scope (default: the projection's LayerNorm), or `params=` directly."""
 
-    def __init__(self, offset=True, params=None):
+    def __init__(self, offset=True, *, params=None, name=ROOT + "projection_shard/~/replicated_layer_norm"):
         self.offset = offset
-        self.params = params            # {"scale": [1, d], "offset": [1, d]}
+        self.params = params if params is not None else _tree(None)[name]
 
     def __call__(self, inputs):
-        L = _abi.lib()
         dev = _dev(inputs)
         x = _f32_in(inputs, dev)
-        d = x.shape[-1]
-        rows = x.reshape(-1, d)
         scale = _f32(torch.as_tensor(self.params["scale"]).to(dev).reshape(-1))
         off = _f32(torch.as_tensor(self.params["offset"]).to(dev).reshape(-1)) if self.offset else torch.zeros_like(scale)
-        out = torch.empty_like(rows)
         with torch.cuda.device(dev):
-            check(L.mtj_layernorm(ptr(rows), ptr(scale), ptr(off), rows.shape[0], d, ptr(out), F32, _abi.stream_handle()))
-        return out.reshape(x.shape)
+            return torch.ops.mtj.layernorm(x, scale, off, 0)
 
 
 class EmbeddingShard:
     """layers.py:165-202 with pe == "rotary" (no positional table)."""
 
-    def __init__(self, config, params, name=None):
+    def __init__(self, config, name=None, *, params=None):
         assert config["n_vocab"] % config.get("cores_per_replica", 1) == 0     # layers.py:172
         self.config = config
-        p = params[ROOT + "embedding_shard/~/linear"]
+        p = _tree(params)[ROOT + "embedding_shard/~/linear"]
         self.w, self.b = p["w"], p["b"]
 
     def __call__(self, x, dtype=None):
-        L = _abi.lib()
         dev = _dev(self.w)
         w = torch.as_tensor(self.w).to(dev)[0].contiguous()
         b = _f32(torch.as_tensor(self.b).to(dev)[0])
         tok = torch.as_tensor(np.asarray(x).astype(np.int32) if not isinstance(x, torch.Tensor) else x.to(torch.int32)).to(dev)
-        tok = tok.reshape(-1).contiguous()
-        out = torch.empty(tok.shape[0], w.shape[1], dtype=torch.float32, device=dev)
         with torch.cuda.device(dev):
-            check(L.mtj_embed(ptr(tok), tok.shape[0], ptr(w), ptr(b), w.shape[0], w.shape[1], _abi.dtype_code(w.dtype),
-                              ptr(out), _abi.stream_handle()))
-        return out
+            return torch.ops.mtj.embed(tok.reshape(-1).contiguous(), w, b)
 
 
 class TransformerLayerShard:
@@ -87,13 +100,13 @@ class TransformerLayerShard:
     slot = position % Tcap), "tokens_decoded": int}.  decode_once updates k and v IN PLACE (the reference
     returns new arrays); the returned dict aliases the same tensors."""
 
-    def __init__(self, config, params, name="layer_0", init_scale=1.0, device="cuda:0"):
+    def __init__(self, config, name=None, init_scale=1.0, *, params=None, device="cuda:0"):
         heads, dim = config["n_heads"], config["d_model"]
         assert dim % heads == 0                                    # layers.py:238
         assert heads % config.get("cores_per_replica", 1) == 0     # layers.py:239
         self.config = config
-        self.index = int(name.split("_")[-1])
-        self.eng = Engine(config, params, device, layer_ids=[self.index], embed=False, proj=False)
+        self.index = int(name.split("_")[-1]) if name else 0      # transformer_shard.py:37: name=f"layer_{i}"
+        self.eng = Engine(config, _tree(params), device, layer_ids=[self.index], embed=False, proj=False)
         self.dim, self.heads, self.dim_per_head = dim, heads, dim // heads
         self.pe_rotary_dims = config.get("pe_rotary_dims", self.dim_per_head)
 
@@ -147,20 +160,13 @@ class TransformerLayerShard:
 class ProjectionShard:
     """layers.py:545-567: final LayerNorm + logits projection (the all_gather is the identity at one shard)."""
 
-    def __init__(self, config, params, name=None, device="cuda:0"):
+    def __init__(self, config, name=None, *, params=None, device="cuda:0"):
         assert config["n_vocab"] % config.get("cores_per_replica", 1) == 0     # layers.py:552
-        self.eng = Engine(config, params, device, layer_ids=[], embed=False, proj=True)
+        self.eng = Engine(config, _tree(params), device, layer_ids=[], embed=False, proj=True)
 
     def __call__(self, x):
-        L = _abi.lib()
         eng, w = self.eng, self.eng.w
         x = _f32_in(x, eng.device).reshape(-1, w.d)
-        M = x.shape[0]
-        out = torch.empty(M, w.V, dtype=torch.float32, device=eng.device)
         with torch.cuda.device(eng.device):
-            s = _abi.stream_handle()
-            h = torch.empty(M, w.d, dtype=w.act_torch_dtype, device=eng.device)
-            check(L.mtj_layernorm(ptr(x), ptr(w.pln_s), ptr(w.pln_o), M, w.d, ptr(h), w.act_dtype, s))
-            check(L.mtj_gemm(ptr(h), w.d, ptr(w.w_p_mm), ptr(w.b_p), M, w.V, w.d, w.mm_dtype, EPI_STORE, ptr(out), w.V, F32,
-                             None, w.alpha_p, s))
-        return out
+            h = torch.ops.mtj.layernorm(x, w.pln_s, w.pln_o, w.act_dtype)
+            return torch.ops.mtj.gemm(h, w.w_p_mm, w.b_p, w.alpha_p, 0)

@@ -6,6 +6,7 @@ per-request top_p / temp, route each completion back to its requester).
 Text handling is pluggable: `encode(str) -> list[int]` and `decode(array) -> str` (e.g. the methods of a locally
 available GPT-2 tokenizer).  Without them requests carry token ids and completions are uint32 arrays.
 """
+import logging
 import queue
 import time
 
@@ -34,63 +35,76 @@ def infer(network, tokens, gen_len=512, top_p=0.9, temp=1.0, top_k=None, seq=Non
     return decode(completion) if decode else completion
 
 
+class _Pending:
+    """One queued request and the queue its completion goes to."""
+    __slots__ = ("prompt", "top_p", "temp", "reply")
+
+    def __init__(self, prompt, top_p, temp):
+        self.prompt, self.top_p, self.temp = prompt, float(top_p), float(temp)
+        self.reply = queue.Queue(maxsize=1)
+
+
 class BatchingLoop:
-    """device_serve.py:138-194.  `submit` is what the request handler does (:54-64); `step` is one turn of the
-    consumer loop; `serve_forever` repeats it."""
+    """The consumer side of the reference's serving script (device_serve.py:138-194) around one generate() call per
+    turn: the batch has a fixed size (the compiled shape there, the recorded HIP graphs here), rows that no request
+    claims run a one-token filler prompt with top_p = temp = 1, every request carries its own top_p / temp, and a
+    request whose prompt cannot be turned into tokens is answered from an empty prompt instead of stopping the loop.
+    `submit` is what a request handler calls (device_serve.py:54-64); `step` serves one batch; `serve_forever` repeats."""
 
-    DUMMY = "whatever"     # the context of the requests that fill a partial batch (device_serve.py:160)
-
-    def __init__(self, network, seq, total_batch, gen_length=256, encode=None, decode=None, poll_s=0.01):
+    def __init__(self, network, seq, total_batch, gen_length=256, encode=None, decode=None, poll_s=0.01, filler=(0,)):
         self.network, self.seq, self.total_batch, self.gen_length = network, seq, total_batch, gen_length
         self.encode, self.decode, self.poll_s = encode, decode, poll_s
-        self.requests_queue = queue.Queue()
+        self.filler = np.asarray(filler, np.int64)
+        self.pending = queue.Queue()
 
     def submit(self, context, top_p, temp):
-        """Queue a request; the completion arrives on the returned queue."""
-        response_queue = queue.Queue()
-        self.requests_queue.put(({"context": context, "top_p": float(top_p), "temp": float(temp)}, response_queue))
-        return response_queue
+        """Queue a request (text, or token ids); its completion arrives on the returned queue."""
+        req = _Pending(context, top_p, temp)
+        self.pending.put(req)
+        return req.reply
 
-    def _tokens(self, ctx):
-        if isinstance(ctx, str):
-            return self.encode(ctx) if self.encode else [0]
-        return ctx
-
-    def step(self, block=True):
-        """Serve up to total_batch pending requests with one generate call; returns how many were served."""
-        all_ctx, all_top_p, all_temp, all_q = [], [], [], []
-        while len(all_ctx) < self.total_batch:
+    def _take(self, block):
+        """Up to total_batch requests, oldest first; waits for the first one when `block`, never for the rest."""
+        batch = []
+        while len(batch) < self.total_batch:
             try:
-                o, q = self.requests_queue.get(block=False)
-                all_ctx.append(o["context"])
-                all_top_p.append(o["top_p"])
-                all_temp.append(o["temp"])
-                all_q.append(q)
+                batch.append(self.pending.get_nowait())
             except queue.Empty:
-                if len(all_ctx) or not block:
+                if batch or not block:
                     break
                 time.sleep(self.poll_s)
-        if not all_ctx:
+        return batch
+
+    def _row(self, prompt):
+        """(padded ids [seq], length) of one prompt; an unusable prompt becomes the empty one."""
+        try:
+            ids = self.encode(prompt) if isinstance(prompt, str) and self.encode else ([0] if isinstance(prompt, str) else prompt)
+            row, n = pad_context(ids, self.seq)
+        except Exception as e:                         # device_serve.py:180-181: the loop outlives a bad request
+            logging.getLogger(__name__).warning("request dropped to an empty prompt: %r", e)
+            row, n = np.zeros(self.seq, np.uint32), 0
+        return row, max(n, 1)
+
+    def step(self, block=True):
+        """Serve the pending requests (at most total_batch) with one generate call; returns how many were served."""
+        batch = self._take(block)
+        if not batch:
             return 0
-        while len(all_ctx) < self.total_batch:          # fill the batch with dummy requests (:159-162)
-            all_ctx.append(self.DUMMY)
-            all_top_p.append(1)
-            all_temp.append(1)
-        all_tokenized, all_length = [], []
-        for ctx in all_ctx:
-            padded_tokens, length = np.zeros(self.seq, np.uint32), 1
-            try:
-                padded_tokens, length = pad_context(self._tokens(ctx), self.seq)
-                length = max(length, 1)
-            except Exception:                            # device_serve.py:180-181: a bad request must not stop the loop
-                print("oops exception")
-            all_tokenized.append(padded_tokens)
-            all_length.append(length)
-        output = self.network.generate(np.array(all_tokenized), np.array(all_length), self.gen_length,
-                                       {"top_p": np.array(all_top_p, np.float64), "temp": np.array(all_temp, np.float64)})
-        for o, q in zip(np.asarray(output[1][0])[:, :, 0], all_q):
-            q.put(self.decode(o) if self.decode else o)
-        return len(all_q)
+        B = self.total_batch
+        ctx = np.zeros((B, self.seq), np.uint32)
+        length = np.ones(B, np.int64)
+        top_p, temp = np.ones(B), np.ones(B)           # rows without a request: top_p = temp = 1 (device_serve.py:159-162)
+        for b in range(B):
+            if b < len(batch):
+                ctx[b], length[b] = self._row(batch[b].prompt)
+                top_p[b], temp[b] = batch[b].top_p, batch[b].temp
+            else:
+                ctx[b], length[b] = self._row(self.filler)
+        out = self.network.generate(ctx, length, self.gen_length, {"top_p": top_p, "temp": temp})
+        tokens = np.asarray(out[1][0])[:, :, 0]
+        for req, row in zip(batch, tokens):
+            req.reply.put(self.decode(row) if self.decode else row)
+        return len(batch)
 
     def serve_forever(self):
         while True:

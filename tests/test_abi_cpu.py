@@ -110,3 +110,15 @@ def test_session_workspace_covers_every_prompt_length():
             assert bound == need, (dtype, M_max, N, K)
     # the case that used to fail: a session first sized for 8 x 599 rows, later used with 8 x 99
     assert lib.mtj_gemm_splitk_work_bytes(8 * 99, 4096, 20480, _abi.F16) > lib.mtj_gemm_splitk_work_bytes(8 * 599, 4096, 20480, _abi.F16)
+
+
+def test_torch_ops_are_registered_for_the_gpu_only():
+    """Every kernel entry point is a dispatcher-visible operator torch.ops.mtj.*; there is no CPU implementation, so
+    host tensors are refused by the dispatcher instead of taking another path."""
+    import torch
+    from mesh_transformer import ops
+    for name in ops.OPS:
+        assert hasattr(torch.ops.mtj, name), name
+    assert "Tensor(a!)" in str(torch.ops.mtj.gemm_resid_.default._schema)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.mtj.layernorm(torch.zeros(2, 8), torch.ones(8), torch.zeros(8), 0)

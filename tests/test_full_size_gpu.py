@@ -42,10 +42,11 @@ def net6b():
 
 
 def test_full_context_forward_agrees_with_the_decode_path(net6b):
-    """Full-context prefill with the 50400-wide projection at every position (16 x 2048 tokens): the logits row of
-    a sequence's last position must agree with the logits the decode path (GEMV kernels, float32 activations,
-    KV-window attention) produces for the same tokens - each path may sit 2e-2 from the exact result, so the two
-    may differ by 4e-2; causality: a row depends on no later token."""
+    """Full-context prefill with the 50400-wide projection at every position (16 x 2048 tokens, BASELINE config 5):
+    the logits row of a sequence's last position must agree within 2e-2 with the logits the decode path (GEMV
+    kernels, float32 activations, KV-window attention) produces for the same tokens (both paths are compared with
+    the oracle itself at this model shape, on shorter inputs, further down); causality: a row depends on no later
+    token."""
     from mesh_transformer import sampling
     rng = np.random.Generator(np.random.Philox(4))
     B, L = 16, 2048
@@ -60,7 +61,7 @@ def test_full_context_forward_agrees_with_the_decode_path(net6b):
     dec = torch.from_numpy(out[2][0, 0, 0]).to(logits.device)
     diff = float((dec - logits[3, L - 1]).abs().max())
     print("max |forward - decode| on the last row:", diff)
-    assert diff < 4e-2
+    assert diff < 2e-2
     # causality: changing the last 100 tokens leaves every earlier row unchanged - bit for bit up to the 32-query
     # group that contains the first changed token (the softmax of a group shares one rescaling decision, so inside
     # that group earlier rows may round differently)
@@ -73,7 +74,7 @@ def test_full_context_forward_agrees_with_the_decode_path(net6b):
     l2 = net6b.forward(np.concatenate([ctx2, ctx[6:8]], 0))
     g0 = first // 32 * 32
     assert torch.equal(l2[0, :g0], keep[:g0])
-    assert float((l2[0, g0:first] - keep[g0:]).abs().max()) < 4e-2
+    assert float((l2[0, g0:first] - keep[g0:]).abs().max()) < 2e-2
     assert float((l2[0, first:] - keep[-1:]).abs().max()) > 0.0
 
 
@@ -99,39 +100,164 @@ def test_batch32_nucleus_decode_rows_are_independent(net6b):
     assert np.array_equal(toks[0], toks[17])
     assert not np.array_equal(toks[4], toks[9])           # same prompt, different uniforms
     # The same two rows alone (batch 2, still the batched kernels, other tile shapes and K ranges in the prefill):
-    # the logits of the first step, whose inputs are the prompt alone, agree as two paths that are each within
-    # 2e-2 of the exact result do.  (The sampled
+    # the logits of the first step, whose inputs are the prompt alone, agree within 2e-2.  (The sampled
     # streams need not: with a flat random-init distribution the nucleus holds thousands of tokens and a logit
     # change of 1e-3 moves the inverse-CDF draw to a neighbour.)
     _, out2 = net6b.generate(ctx[[0, 4]], [P, P], 2, {"top_p": np.full(2, 0.9), "temp": np.full(2, 0.8)},
                              uniforms=u[[0, 4], :2], return_logits=True)
     d = np.abs(out2[2][:, 0, 0] - out[2][[0, 4], 0, 0]).max()
     print("first-step logits, batch 2 against batch 32: max |d|", d)
-    assert d < 4e-2
+    assert d < 2e-2
 
 
-def test_decode_against_the_committed_6b_oracle_run():
-    """The CPU oracle's own run at the full 6B shape (tests/golden/gptj6b_decode.npz, written by
-    tests/golden/make_golden_6b.py: float32 arithmetic on the bf16 hashed synthetic tree, 128-token prompt, 8 greedy
-    steps): |dlogit| <= 2e-2 on every stored logit and the same greedy tokens."""
+GOLDEN = None
+
+
+def golden(name):
     import os
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name))
+
+
+@pytest.fixture(scope="module")
+def net_hashed():
+    """The full 6B model on the hashed synthetic tree the oracle's fixtures were computed on (same bits on any device)."""
     from oracle import gptj_oracle as O
     from mesh_transformer import sampling
     from mesh_transformer.transformer_shard import CausalTransformer
-    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gptj6b_decode.npz"))
     dev = torch.device("cuda:0")
-    tree = O.hashed_params(CFG_6B, int(g["seed"]), torch.bfloat16, device=dev)
-    net = CausalTransformer(dict(CFG_6B, sampler=sampling.greedy_sample), tree)
-    prompt = g["prompt"]
-    G = len(g["tokens"])
-    _, out = net.generate(prompt, [prompt.shape[1]], G, {}, return_logits=True)
-    lg = out[2][0, :, 0]                                            # [G, V]
+    seed = int(golden("gptj6b_decode.npz")["seed"])
+    net = CausalTransformer(dict(CFG_6B, sampler=sampling.greedy_sample), O.hashed_params(CFG_6B, seed, torch.bfloat16, device=dev))
+    yield net
+    del net
+    torch.cuda.empty_cache()
+
+
+def logit_errors(lg, g):
+    """max |dlogit| of rows lg [R, V] against the stored subset of the oracle's rows: every 50th logit and the top 32"""
     stride = int(g["stride"])
     e1 = np.abs(lg[:, ::stride] - g["strided_logits"]).max()
     e2 = np.abs(np.take_along_axis(lg, g["top_ids"].astype(np.int64), -1) - g["top_logits"]).max()
-    print("6B decode vs the oracle's run: max |dlogit| strided", e1, "top-32", e2)
-    assert e1 < 2e-2 and e2 < 2e-2
-    assert np.abs(lg.astype(np.float64).sum(-1) - g["logit_sum"]).max() < 2e-2 * lg.shape[1] ** 0.5 * 4
-    assert np.array_equal(out[0][0, :, 0].astype(np.int64), g["tokens"])
-    del net, tree
+    return float(e1), float(e2)
+
+
+TOL_6B = 2e-2     # north-star bound on the logits of the bf16 model against the float32-activation reference
+
+
+def test_decode_against_the_committed_6b_oracle_run(net_hashed):
+    """BASELINE config 3 shape against the oracle's own run (tests/golden/gptj6b_decode.npz, written by
+    tests/golden/make_golden_6b.py: float32 arithmetic on the bf16 hashed tree): a 512-token prompt left-padded to
+    576 - its 511-token prefill runs on the 256x256 matrix-core kernel - and 32 greedy steps.
+    (1) teacher-forced (the oracle's tokens fed back through a host sampler): |dlogit| <= 2e-2 on every stored logit
+    of all 32 steps, and the argmax agrees wherever the oracle's top-1/top-2 margin exceeds twice the measured error;
+    (2) free-running on the device (HIP-graph replay): the same tokens for as long as every choice of the oracle is
+    decided by a margin of 0.03 (the stored margins say how long that is)."""
+    g = golden("gptj6b_decode.npz")
+    ctx, P, want = g["ctx"], [int(g["ctx_length"][0])], g["tokens"]
+    G = len(want)
+    step = {"t": 0}
+
+    def teacher(key, logits, sampler_input, **kw):
+        t = step["t"]
+        step["t"] += 1
+        return np.asarray([want[t]], np.uint32), None
+
+    _, out = net_hashed.generate(ctx, P, G, {}, return_logits=True, sampler=teacher)
+    lg = out[2][0, :, 0]
+    e1, e2 = logit_errors(lg, g)
+    print("6B decode, teacher-forced, vs the oracle: max |dlogit| strided", e1, "top-32", e2)
+    assert e1 < TOL_6B and e2 < TOL_6B
+    assert np.abs(lg.astype(np.float64).sum(-1) - g["logit_sum"]).max() < TOL_6B * lg.shape[1] ** 0.5 * 4
+    decided = g["margins"] > 2 * max(e1, e2)
+    assert np.array_equal(lg.argmax(-1)[decided], want[decided])
+    clear = g["margins"] >= 0.03
+    n_clear = G if clear.all() else int(np.argmin(clear))
+    print("oracle margins: smallest", float(g["margins"].min()), "- free-running stream compared for", n_clear, "steps")
+    _, out2 = net_hashed.generate(ctx, P, G, {})
+    assert np.array_equal(out2[0][0, :n_clear, 0].astype(np.int64), want[:n_clear])
+
+
+def test_every_position_forward_and_eval_against_the_6b_oracle(net_hashed):
+    """The every-position logits of a 128-token forward at the full 6B shape (the path of BASELINE config 5: matrix-core
+    GEMMs and flash attention end to end) within 2e-2 of the oracle's on every stored logit of every position, and
+    the evaluation losses computed from them (ProjectionShard.loss, layers.py:569-593)."""
+    g = golden("gptj6b_forward.npz")
+    ctx = g["ctx"]
+    lg = net_hashed.forward(ctx)[0].cpu().numpy()
+    e1, e2 = logit_errors(lg, g)
+    print("6B forward, 128 positions, vs the oracle: max |dlogit| strided", e1, "top-32", e2)
+    assert e1 < TOL_6B and e2 < TOL_6B
+    res = net_hashed.eval({"obs": ctx, "target": g["target"]})
+    err = np.abs(res["all_loss"][0] - g["all_loss"]).max()
+    print("6B eval: max |dloss|", float(err))
+    assert err < TOL_6B
+    sure = g["target_margin"] > 2 * TOL_6B          # positions where 'target holds the maximum' is not a near-tie
+    assert np.array_equal(res["correct"][0][sure], g["correct"][sure])
+
+
+def test_batch2_decode_against_the_6b_oracle(net_hashed):
+    """Batched decode (the matrix-core decode path of BASELINE config 4) at the full 6B shape: two ragged prompts,
+    8 greedy steps, logits of every step within 2e-2 of the oracle's and the same tokens (every choice of the
+    oracle's runs is decided by a margin above 0.03)."""
+    g = golden("gptj6b_batch2.npz")
+    ctx, lens, want = g["ctx"], g["ctx_length"].tolist(), g["tokens"]
+    G = want.shape[1]
+    _, out = net_hashed.generate(ctx, lens, G, {}, return_logits=True)
+    for b in range(2):
+        gb = {k: (g[k][b] if g[k].ndim and k != "stride" else g[k]) for k in ("strided_logits", "top_ids", "top_logits", "stride")}
+        e1, e2 = logit_errors(out[2][b, :, 0], gb)
+        print(f"6B batch-2 decode row {b} vs the oracle: max |dlogit| strided", e1, "top-32", e2)
+        assert e1 < TOL_6B and e2 < TOL_6B
+    assert float(g["margins"].min()) >= 0.03
+    assert np.array_equal(out[0][:, :, 0].astype(np.int64), want)
+    _, out2 = net_hashed.generate(ctx, lens, G, {})       # HIP-graph replay
+    assert np.array_equal(out2[0], out[0])
+
+
+def test_session_reuse_with_a_shorter_prompt(net_hashed):
+    """A session sized by a long prompt is reused for a short one on the same (batch, window): the out projection of
+    the short prefill is cut into more K ranges and needs MORE split-K workspace than the long one did."""
+    from oracle import gptj_oracle as O
+    B, L = 2, 700
+    long_ctx = O.left_pad(O.seeded_prompt(31, B, 600), L)
+    short_ctx = O.left_pad(O.seeded_prompt(32, B, 100), L)
+    net_hashed.generate(long_ctx, [600, 600], 2, {})
+    _, warm = net_hashed.generate(short_ctx, [100, 100], 4, {}, return_logits=True)
+    net_hashed.engine().sessions.pop((B, L - 1), None)
+    _, cold = net_hashed.generate(short_ctx, [100, 100], 4, {}, return_logits=True)
+    assert np.array_equal(warm[0], cold[0]) and np.array_equal(warm[2], cold[2])
+
+
+def test_config2_one_full_shape_layer_against_the_float32_reference_layer():
+    """BASELINE config 2: one layer of the 6B shape, bf16 weights ~N(0, 0.02) seed 1, activations [8, 2048, 4096]
+    ~N(0, 1).  The HIP layer (LayerNorm, fused q|v|k|fc_in GEMM with RoPE and GELU, flash attention, out|fc_out GEMM
+    with the residual add, all on the 256x256 matrix-core kernel) against TransformerLayerShard.__call__
+    (layers.py:299-313) evaluated by the CPU oracle in float32 on two of the eight sequences."""
+    from oracle import gptj_oracle as O
+    from mesh_transformer.engine import Engine
+    dev = torch.device("cuda:0")
+    cfg = dict(layers=1, d_model=4096, n_heads=16, n_vocab=64, norm="layernorm", pe="rotary", pe_rotary_dims=64,
+               cores_per_replica=1)
+    p = O.seeded_params(cfg, 1, torch.bfloat16)
+    eng = Engine(cfg, {k: {n: v.to(dev) for n, v in m.items()} for k, m in p.items()}, dev, layer_ids=[0], embed=False, proj=False)
+    B, T, d = 8, 2048, 4096
+    x_host = torch.randn(B, T, d, generator=torch.Generator().manual_seed(1))
+    x = x_host.reshape(B * T, d).to(dev)
+    x0 = x.clone()
+    ses = eng.session(B, T, T, T + 8)
+    pos0 = torch.zeros(B, dtype=torch.int32, device=dev)
+    eng.layer_prefill(ses, 0, x, ses.h_pf[:B * T], ses.act_pf[:B * T], T, pos0)
+    torch.cuda.synchronize()
+    delta = (x - x0).reshape(B, T, d)
+    layer = O.Layer(cfg, p, 0, torch.float32)
+    torch.set_num_threads(max(torch.get_num_threads(), 16))
+    for b in (0, 5):
+        ref = layer(x_host[b], 0.0)
+        got = delta[b].cpu()
+        rel = float((got.double() - ref.double()).norm() / ref.double().norm())
+        worst = float((got.double() - ref.double()).abs().max())
+        print(f"config 2, sequence {b}: relative error of the layer output {rel:.3e}, max abs {worst:.3e} (output std {float(ref.std()):.3f})")
+        assert rel < 1e-3
+        row = (got.double() - ref.double()).norm(dim=1) / ref.double().norm(dim=1)
+        assert float(row.max()) < 4e-3, int(row.argmax())
+    del eng
     torch.cuda.empty_cache()

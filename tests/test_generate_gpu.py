@@ -32,18 +32,21 @@ def net_for(cfg, params, sampler):
 
 def test_config1_layers_fp32_within_1e4_relative():
     """Per-layer bound of the float32 path: prefill (left-padded) and one decode step of every layer."""
+    from mesh_transformer import layers
     from mesh_transformer.layers import TransformerLayerShard, EmbeddingShard, ProjectionShard, ReplicatedLayerNorm
     params = O.seeded_params(CFG1, 0)
+    scope = layers.transform(params)          # the modules take their parameters from the enclosing scope, like haiku's
+    scope.__enter__()
     model = O.Model(CFG1, params, torch.float64)
     prompt = O.seeded_prompt(0, 1, 128)
     ctx = O.left_pad(prompt, 168)[0]
     T, given = 167, 127
     x_ref = model.embed(ctx[:-1])
-    emb = EmbeddingShard(CFG1, params)(ctx[:-1])
+    emb = EmbeddingShard(CFG1)(ctx[:-1])
     assert rel(emb, x_ref) < 1e-6
     x_new_ref = model.embed(ctx[-1:])
     for i, lref in enumerate(model.layers):
-        layer = TransformerLayerShard(CFG1, params, name=f"layer_{i}")
+        layer = TransformerLayerShard(CFG1, f"layer_{i}", 2.0 / CFG1["layers"])     # transformer_shard.py:35-37
         d_ref, st_ref = lref.get_init_decode_state(x_ref, given, 0.0)
         d_got, st = layer.get_init_decode_state(x_ref.float(), given, 0)
         pad = T - given
@@ -62,10 +65,15 @@ def test_config1_layers_fp32_within_1e4_relative():
         assert e < 1e-4 and st2["tokens_decoded"] == given + 1
         x_ref = x_ref + d_ref
         x_new_ref = x_new_ref + dd_ref
-    lg = ProjectionShard(CFG1, params)(x_new_ref.float())
+    lg = ProjectionShard(CFG1)(x_new_ref.float())
     assert rel(lg, model.proj(x_new_ref)) < 1e-4
+    ln = ReplicatedLayerNorm()(x_new_ref.float())
+    assert rel(ln, O.replicated_layer_norm(x_new_ref, model.pln_s, model.pln_o)) < 1e-5
     ln = ReplicatedLayerNorm(params=params[O.PROJ_LN])(x_new_ref.float())
     assert rel(ln, O.replicated_layer_norm(x_new_ref, model.pln_s, model.pln_o)) < 1e-5
+    scope.__exit__(None, None, None)
+    with pytest.raises(RuntimeError):
+        EmbeddingShard(CFG1)                  # no parameters in scope
 
 
 def test_config1_generate_fp32_greedy_stream():
@@ -227,6 +235,31 @@ def test_batching_loop_on_the_gpu():
     for p, q in zip(prompts, qs):
         ref = m.generate(O.left_pad(p[None], 40), [len(p)], 6, O.greedy_sample, {})
         assert np.array_equal(q.get_nowait(), ref[0][0, :, 0])
+
+
+def test_infer_on_the_gpu_against_the_oracle():
+    """The single-prompt caller of resharding_example.py:55-75 / device_sample.py:86-103 (pad to seq, generate with
+    top_p / temp / top_k, index output[1][0][0, :, 0]) through the real network.  With top_p -> 0 the nucleus is the
+    top token alone (top_k = 5 on top of it changes nothing: the reference's top-k spares token 0, sampling.py:15-26,
+    but top_p removes it), so with the uniforms drawn inside generate the completion is the oracle's nucleus run on
+    ANY uniforms; a prompt longer than seq keeps its last seq tokens."""
+    from mesh_transformer import sampling, serving
+    cfg = dict(CFG1, n_vocab=2048, seq=48)
+    params = O.seeded_params(cfg, 13)
+    net = net_for(cfg, params, sampling.nucleaus_sample)
+    m = O.Model(cfg, params, torch.float64)
+    for n in (17, 60):
+        prompt = O.seeded_prompt(40 + n, 1, n, hi=2048)[0]
+        got = serving.infer(net, prompt.tolist(), gen_len=7, top_p=1e-9, temp=0.7, top_k=5)
+        kept = prompt[-48:]
+        ctx = O.left_pad(kept[None], 48)
+        opts = {"top_p": np.array([1e-9]), "temp": np.array([0.7]), "top_k": np.array([5])}
+        ref = m.generate(ctx, [len(kept)], 7, O.nucleaus_sample, opts, uniforms=np.full((1, 7), 0.37))
+        ref2 = m.generate(ctx, [len(kept)], 7, O.nucleaus_sample, opts, uniforms=np.full((1, 7), 0.93))
+        assert np.array_equal(ref[0], ref2[0])                       # the draw has one reachable token
+        assert got.dtype == np.uint32 and np.array_equal(got, ref[0][0, :, 0]), n
+    text = serving.infer(net, [5, 6, 7], gen_len=3, top_p=1e-9, decode=lambda a: " ".join(str(int(t)) for t in a))
+    assert len(text.split()) == 3
 
 
 def test_generate_from_an_8_shard_checkpoint(tmp_path):

@@ -589,6 +589,56 @@ def test_attn_decode_partials_merged_by_the_out_projection_gemv(L, dt, dh, H, F,
     assert rel_err(x, ref) < 5e-6, (dt, dh, Tcap, p)
 
 
+# ------------------------------------------------------------------ the same kernels as torch.ops.mtj operators
+def test_torch_ops_reach_the_same_kernels():
+    from mesh_transformer import ops  # noqa: F401
+    g = torch.Generator().manual_seed(5)
+    M, K, N = 70, 256, 192
+    x = torch.randn(M, K, generator=g).to(DEV)
+    sc, of = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV), (0.1 * torch.randn(K, generator=g)).to(DEV)
+    h = torch.ops.mtj.layernorm(x, sc, of, 0)
+    ref = O.replicated_layer_norm(x.double().cpu(), sc.double().cpu(), of.double().cpu())
+    assert rel_err(h, ref) < 3e-6
+    h16 = torch.ops.mtj.layernorm(x, sc, of, 2)
+    assert h16.dtype == torch.float16 and rel_err(h16, ref) < 5e-4
+    Wh = (torch.randn(K, N, generator=g) * 0.05).to(torch.bfloat16).to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    W16 = torch.ops.mtj.pack_weight_f16(Wh, 64.0)
+    y = torch.ops.mtj.gemm(h16, W16, bias, 1.0 / 64.0, 0)
+    assert rel_err(y, h16.double() @ Wh.double() + bias.double()) < 5e-6
+    x2 = torch.randn(M, N, generator=g).to(DEV)
+    x2_0 = x2.clone()
+    torch.ops.mtj.gemm_resid_(x2, h16, W16, bias, 1.0 / 64.0)
+    assert rel_err(x2, x2_0.double() + h16.double() @ Wh.double() + bias.double()) < 5e-6
+    Wp = torch.ops.mtj.pack_weight(Wh)
+    assert torch.equal(Wp, Wh.T.contiguous())
+    v = torch.ops.mtj.gemv(x[0].contiguous(), Wp, bias, sc, of)
+    assert rel_err(v, ref[0].to(DEV) @ Wh.double() + bias.double()) < 6e-6
+    # one-token attention, embedding, cross entropy, samplers
+    B, H, Tcap, dh = 2, 4, 50, 64
+    q = torch.randn(B, H, dh, generator=g).to(DEV)
+    kc = torch.randn(B, H, Tcap, dh, generator=g).to(torch.float16).to(DEV)
+    vc = torch.randn(B, H, Tcap, dh, generator=g).to(torch.float16).to(DEV)
+    pos = torch.tensor([10, 70], dtype=torch.int32, device=DEV)
+    o = torch.ops.mtj.attn_decode(q, kc, vc, pos, 0)
+    for b, p in enumerate([10, 70]):
+        n = min(p + 1, Tcap)
+        s_ = torch.einsum("hd,hTd->hT", q[b].double(), kc[b, :, :n].double()) / math.sqrt(dh)
+        assert rel_err(o[b], torch.einsum("hT,hTd->hd", torch.softmax(s_, -1), vc[b, :, :n].double()).reshape(-1)) < 3e-6
+    We = torch.randn(100, 32, generator=g).to(DEV)
+    tok = torch.tensor([3, 99], dtype=torch.int32, device=DEV)
+    assert torch.equal(torch.ops.mtj.embed(tok, We, bias[:32].contiguous()), We[tok.long()] + bias[:32])
+    lg = torch.randn(5, 300, generator=g).to(DEV)
+    tgt = torch.tensor([1, 299, 7, 0, 150], dtype=torch.int32, device=DEV)
+    loss, correct = torch.ops.mtj.xent(lg, tgt)
+    assert rel_err(loss, torch.nn.functional.cross_entropy(lg.double(), tgt.long(), reduction="none")) < 1e-6
+    assert torch.equal(torch.ops.mtj.sample_greedy(lg).long(), lg.argmax(-1))
+    f64 = lambda v: torch.full((5,), v, dtype=torch.float64, device=DEV)
+    t, filt, keep = torch.ops.mtj.sample_nucleus(lg, f64(0.5), f64(1.0), None, f64(0.3))
+    want = O.nucleaus_filter(lg.cpu().numpy(), 0.5)
+    assert np.array_equal(filt.cpu().numpy(), want) and np.array_equal(keep.cpu().numpy(), want == lg.cpu().numpy())
+
+
 # ------------------------------------------------------------------ samplers: bit-exact against the oracle
 def _sample(L, logits, top_p, temp, top_k, u):
     a = abi()

@@ -163,6 +163,25 @@ int mtj_gemv(const float* x, const float* ln_scale, const float* ln_offset, cons
              int64_t N, int64_t K, int dtype, int epi, void* out, int out_dtype, const mtj_inproj* ip,
              const mtj_attn_merge* am, void* stream);
 
+/* The out projection of a batch-1 decode layer with the one-token attention inside it (layers.py:275-285, 290, 313,
+ * 316-344): out[N] += [attention(q, K/V window) | x[H*dh .. K)] @ W^T + bias, float32 in place.  The first workgroups
+ * reduce the key ranges of the heads to partials while the weight stream of the launch starts; every workgroup
+ * streams the columns of its rows that do not depend on the attention first, then waits (on an arrival counter in
+ * `work`) for all partials, merges them and finishes its rows.  Compared with mtj_attn_decode_partials + mtj_gemv it
+ * saves a launch and the exposed round trips of the attention.
+ * Needs every workgroup resident at once: mtj_gemv_attn_supported() says whether the shape qualifies on the current
+ * device (whole 8 KiB tiles on both sides of column H*dh, at most one workgroup per CU); MTJ_ELIMIT otherwise.
+ * x float32 [K] (its first H*dh entries are not read); q float32 [H, dh]; caches [H, Tcap, dh] in kv_dtype; pos
+ * int32 [1].  `work`: mtj_gemv_attn_work_bytes(H, dh) bytes, 128-byte aligned, zeroed by the caller ONCE before its
+ * first use and then left alone (it holds a running arrival counter); launches sharing one `work` must not overlap
+ * and must all have the same N.  Word 2 of `work` becomes non-zero if a launch ever gave up waiting (its result is
+ * then unusable). */
+int mtj_gemv_attn_supported(int64_t N, int64_t K, int dtype, int64_t H, int64_t dh, int kv_dtype, int64_t Tcap);
+int64_t mtj_gemv_attn_work_bytes(int64_t H, int64_t dh);
+int mtj_gemv_attn(const float* x, const void* W, const float* bias, int64_t N, int64_t K, int dtype, float* out,
+                  const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t H, int64_t Tcap,
+                  int64_t dh, int kv_dtype, void* work, void* stream);
+
 /* Causal self-attention over a left-padded rectangle (self_attn + masks of get_init_decode_state,
  * layers.py:260-285, 347-366).  q [B,H,Tp,dh], k_cache [B,H,Tcap,dh] (rotated), v_t [B,H,dh,ldvt] with
  * ldvt >= Tp rounded up to a multiple of 64 (columns beyond the last key may hold anything);

@@ -361,28 +361,6 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
 constexpr int DEC_NI = 8;            // K (and V) loads per lane and step
 constexpr int DEC_PAD = MTJ_DEC_PAD;  // floats in front of the vector of a partial
 
-template <typename T> struct kvrow;   // one 16-byte piece of a cached row -> EPC floats
-template <> struct kvrow<float> {
-  static constexpr int EPC = 4;
-  __device__ static __forceinline__ void get(const uint32x4& w, float* f) {
-    f[0] = __uint_as_float(w.x); f[1] = __uint_as_float(w.y); f[2] = __uint_as_float(w.z); f[3] = __uint_as_float(w.w);
-  }
-};
-template <> struct kvrow<bf16_t> {
-  static constexpr int EPC = 8;
-  __device__ static __forceinline__ void get(const uint32x4& w, float* f) {
-    f[0] = bf16_lo(w.x); f[1] = bf16_hi(w.x); f[2] = bf16_lo(w.y); f[3] = bf16_hi(w.y);
-    f[4] = bf16_lo(w.z); f[5] = bf16_hi(w.z); f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
-  }
-};
-template <> struct kvrow<f16_t> {
-  static constexpr int EPC = 8;
-  __device__ static __forceinline__ void get(const uint32x4& w, float* f) {
-    f[0] = f16_lo(w.x); f[1] = f16_hi(w.x); f[2] = f16_lo(w.y); f[3] = f16_hi(w.y);
-    f[4] = f16_lo(w.z); f[5] = f16_hi(w.z); f[6] = f16_lo(w.w); f[7] = f16_hi(w.w);
-  }
-};
-
 template <typename T, int DH>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const T* __restrict__ kc,
                                                           const T* __restrict__ vc, const int32_t* __restrict__ pos,
@@ -509,7 +487,7 @@ __global__ __launch_bounds__(DH / 4) void attn_combine_kernel(const float* __res
                                                               void* __restrict__ out, int64_t ld_out, int out_dtype) {
   const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int64_t bh = (int64_t)b * H + h;
-  const floatx4 a = mtj_merge_partials(work + bh * S * (DH + DEC_PAD), S, DH, 4 * tid);
+  const floatx4 a = mtj_merge_partials(work + bh * S * (DH + DEC_PAD), S, DH + DEC_PAD, 4 * tid);
   const int64_t o = (int64_t)b * ld_out + h * DH + 4 * tid;
   store_as(out, o, a.x, out_dtype);
   store_as(out, o + 1, a.y, out_dtype);

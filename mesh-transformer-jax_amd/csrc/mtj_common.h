@@ -154,15 +154,38 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// ---------------------------------------------------------------- cached K/V rows
+template <typename T> struct kvrow;   // one 16-byte piece of a cached row -> EPC floats
+template <> struct kvrow<float> {
+  static constexpr int EPC = 4;
+  __device__ static __forceinline__ void get(const uint32x4& w, float* f) {
+    f[0] = __uint_as_float(w.x); f[1] = __uint_as_float(w.y); f[2] = __uint_as_float(w.z); f[3] = __uint_as_float(w.w);
+  }
+};
+template <> struct kvrow<bf16_t> {
+  static constexpr int EPC = 8;
+  __device__ static __forceinline__ void get(const uint32x4& w, float* f) {
+    f[0] = bf16_lo(w.x); f[1] = bf16_hi(w.x); f[2] = bf16_lo(w.y); f[3] = bf16_hi(w.y);
+    f[4] = bf16_lo(w.z); f[5] = bf16_hi(w.z); f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
+  }
+};
+template <> struct kvrow<f16_t> {
+  static constexpr int EPC = 8;
+  __device__ static __forceinline__ void get(const uint32x4& w, float* f) {
+    f[0] = f16_lo(w.x); f[1] = f16_hi(w.x); f[2] = f16_lo(w.y); f[3] = f16_hi(w.y);
+    f[4] = f16_lo(w.z); f[5] = f16_hi(w.z); f[6] = f16_lo(w.w); f[7] = f16_hi(w.w);
+  }
+};
+
 // ---------------------------------------------------------------- merge of one-token attention partials
-// Partials of one (sequence, head): wb[s * (dh + MTJ_DEC_PAD)] = {max, sum, -, -, V[dh]} for key range s < S <= 8.
+// Partials of one (sequence, head): wb[s * stride] = {max, sum, -, -, V[dh]} for key range s < S <= 8.
 // Returns elements e .. e+3 of sum_s exp(max_s - max) V_s / sum_s exp(max_s - max) sum_s.  The ranges are taken four at
 // a time with a running maximum (four vectors and eight statistics in registers at once: the callers have their
 // weight tiles in registers too); inside a batch every load is issued before the first is used.  Ranges beyond S
 // read range S-1 again with weight 0.
 constexpr int MTJ_DEC_MAXS = 8;
 constexpr int MTJ_DEC_PAD = 4;
-__device__ __forceinline__ floatx4 mtj_merge_partials(const float* __restrict__ wb, int S, int dh, int e) {
+__device__ __forceinline__ floatx4 mtj_merge_partials(const float* __restrict__ wb, int S, int stride, int e) {
   float mm = -INFINITY, lt = 0.f;
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int s0 = 0; s0 < S; s0 += 4) {
@@ -170,7 +193,7 @@ __device__ __forceinline__ floatx4 mtj_merge_partials(const float* __restrict__ 
     floatx4 v[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float* p = wb + (int64_t)(s0 + i < S ? s0 + i : S - 1) * (dh + MTJ_DEC_PAD);
+      const float* p = wb + (int64_t)(s0 + i < S ? s0 + i : S - 1) * stride;
       m[i] = p[0];
       l[i] = p[1];
       v[i] = *reinterpret_cast<const floatx4*>(p + MTJ_DEC_PAD + e);

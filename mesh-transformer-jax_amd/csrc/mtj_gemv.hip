@@ -179,7 +179,8 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
     for (int k = tid * 4; k < dm; k += blockDim.x * 4) {
       const int h = k / a.am.d_head, e = k - h * a.am.d_head;
       *reinterpret_cast<floatx4*>(xs + k) =
-          mtj_merge_partials(a.am.partials + (int64_t)h * a.am.splits * (a.am.d_head + MTJ_DEC_PAD), a.am.splits, a.am.d_head, e);
+          mtj_merge_partials(a.am.partials + (int64_t)h * a.am.splits * (a.am.d_head + MTJ_DEC_PAD), a.am.splits,
+                             a.am.d_head + MTJ_DEC_PAD, e);
     }
     for (int k = dm + tid * 4; k < K; k += blockDim.x * 4)
       *reinterpret_cast<floatx4*>(xs + k) = *reinterpret_cast<const floatx4*>(a.x + k);
@@ -275,6 +276,286 @@ int launch(const gemv_args& a, hipStream_t s) {
   return mtj_check_launch("mtj_gemv");
 }
 
+// ------------------------------------------------------------------------------------------------
+// Out projection of a decode layer with the one-token attention inside it:  x += [attention | gelu] @ W_out^T + b.
+//
+// The attention output is only the first H*dh of the K inputs, so the kernel streams the other columns of its rows
+// first and needs the attention result only for the last tile(s) of every row.  The attention itself is spread over
+// the first H*S workgroups - workgroup b reduces key range b % S of head b / S to a partial (max, sum, weighted V), as
+// attn_decode_kernel does - right after the first weight tiles have been requested, so its loads travel with the weight
+// stream.  The partials go to memory with agent-scope stores, every workgroup then bumps an arrival counter, and just
+// before the attention columns are due (some 20 us later at the 6B shape) a workgroup waits until all arrivals of
+// this launch are in, merges the S partials of every head into its copy of the input vector and finishes its rows.
+// One launch instead of attention launch + merge.  Measured at the 6B shape, 650 keys (33.3 us against 30.6 + 6.5):
+// the workgroups with a key range run ~3.5 us behind the others from the start (their K/V rows compete with the 32 MB
+// of first weight tiles that the whole grid requests at once, whichever is asked for first) and their arrival
+// costs another ~5 us (agent-scope stores are acknowledged by memory, not by the L2), both hidden behind the ~17 us
+// of the first pass; exposed are the merge (two batches of four partials, ~2.8 us) and the pipeline drain.
+//
+// The wait needs every workgroup of the grid to be resident at once: the host launches at most one workgroup per
+// CU.  The spin is bounded; if it ever gave up, word 2 of the counter block is set and the result is unusable.
+// Counter block: work[0] 64-bit arrival counter (never reset: a launch's target is the next multiple of the grid
+// size above the value its own arrival returned; the caller zeroes `work` once), then the partials, one per
+// (head, range), each in its own 128-byte lines so that no line is shared between writers of different L2s.
+constexpr int OA_NI = 4;              // K (and V) loads per lane and attention step: 128 keys of d_head 256 per workgroup
+constexpr int OA_HEAD = 32;           // floats in front of the partials (counter block)
+
+struct outatt_args {
+  gemv_args g;                         // x (entries [0, H*dh) unused), W, bias, N, K, out (residual, in place)
+  const float* q;                      // [H, dh]
+  const void* kc;
+  const void* vc;
+  const int32_t* pos;
+  int H, Tcap, S;
+  float* work;
+};
+
+__device__ __forceinline__ int oa_pstride(int dh) { return (dh + MTJ_DEC_PAD + 31) / 32 * 32; }
+
+template <typename T, typename TKV, int DH>
+__global__ __launch_bounds__(1024) void gemv_outatt_kernel(const outatt_args oa) {
+  const gemv_args& a = oa.g;
+  extern __shared__ __align__(16) float xs[];                 // K floats
+  __shared__ float part[16][DH];
+  __shared__ float stat[16][2];
+  constexpr int EPC = chunk<T>::EPC;
+  constexpr int STEP = 64 * EPC;
+  constexpr int U = 8;
+  constexpr int TILE = STEP * U;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int K = (int)a.K;
+  const T* __restrict__ W = reinterpret_cast<const T*>(a.W);
+  const int dm = oa.H * DH;                                    // inputs that come from the attention
+  const int ta = dm / TILE, tpr = K / TILE;                    // tiles of a row: [0, ta) attention, [ta, tpr) the rest
+  const int nwg = gridDim.x;
+
+  // rows of this wavefront: as in gemv_kernel
+  const int64_t ub0 = a.N * blockIdx.x / nwg, ub1 = a.N * (blockIdx.x + 1) / nwg;
+  const int cnt = (int)(ub1 - ub0), per = cnt / 16, rem = cnt % 16;
+  const int64_t row0 = ub0 + (int64_t)wave * per + (wave < rem ? wave : rem);
+  const int nrows = per + (wave < rem ? 1 : 0);
+
+  const int p = oa.pos[0];
+  float pre_add = 0.f;
+  if (lane < nrows) {
+    const int64_t n = row0 + lane;
+    pre_add = (a.bias ? a.bias[n] : 0.f) + reinterpret_cast<const float*>(a.out)[n];
+  }
+  // tile number i of the first pass is tile ta + i % (tpr - ta) of row i / (tpr - ta); of the second pass tile i % ta of
+  // row i / ta.  A wavefront without rows reads (and drops) row 0.
+  const T* base = W + (nrows > 0 ? row0 : 0) * a.K + lane * EPC;
+  const int n1 = nrows * (tpr - ta), n2 = nrows * ta;
+  auto request = [&](uint32x4 (&t)[U], int i, int t0, int tn) {
+    const int r = i / tn, tt = t0 + i - r * tn;
+    const T* src = base + (int64_t)r * K + tt * TILE;
+#pragma unroll
+    for (int u = 0; u < U; ++u) t[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(src + u * STEP));
+  };
+  uint32x4 w[U], w2[U];
+
+  // ---- attention: requests
+  constexpr int KEPC = kvrow<TKV>::EPC;
+  constexpr int LPK = DH / KEPC, KPL = 64 / LPK, NI = OA_NI;
+  constexpr int ASTEP = 16 * NI * KPL;                         // keys per workgroup step
+  const int S = oa.S;
+  const bool has_att = (int)blockIdx.x < oa.H * S;
+  const int h = blockIdx.x / S, split = blockIdx.x - h * S;
+  const int nvalid = (p + 1 < oa.Tcap) ? p + 1 : oa.Tcap;
+  const int kper = (nvalid + S - 1) / S;
+  const int k0 = split * kper;
+  const int nk = !has_att ? 0 : (k0 + kper <= nvalid) ? kper : nvalid - k0;
+  const int sub = lane / LPK, el = (lane % LPK) * KEPC;
+  const TKV* kbase = reinterpret_cast<const TKV*>(oa.kc) + ((int64_t)h * oa.Tcap + k0) * DH + el;
+  const TKV* vbase = reinterpret_cast<const TKV*>(oa.vc) + ((int64_t)h * oa.Tcap + k0) * DH + el;
+  uint32x4 kr[NI], vr[NI];
+  auto att_request = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      int kk = kb + (i * 16 + wave) * KPL + sub;
+      kk = kk < nk ? kk : nk - 1;
+      kr[i] = *reinterpret_cast<const uint32x4*>(kbase + (int64_t)kk * DH);
+      vr[i] = *reinterpret_cast<const uint32x4*>(vbase + (int64_t)kk * DH);
+    }
+  };
+  // a workgroup with a key range asks for its K/V rows first, so that they do not queue behind 8 KiB of weights
+  // per wavefront (loads return in the order they were issued)
+  float qv[KEPC];
+  if (nk > 0) {
+    att_request(0);
+#pragma unroll
+    for (int j = 0; j < KEPC; ++j) qv[j] = oa.q[h * DH + el + j];
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  request(w, 0, ta, tpr - ta);                                 // n1 >= 1 whenever nrows >= 1; harmless otherwise
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- stage the inputs that do not come from the attention
+  for (int k = dm + tid * 4; k < K; k += 4096)
+    *reinterpret_cast<floatx4*>(xs + k) = *reinterpret_cast<const floatx4*>(a.x + k);
+
+  // ---- attention: reduce my key range
+  float m_run = -INFINITY, l_run = 0.f;
+  float acc_a[KEPC];
+#pragma unroll
+  for (int j = 0; j < KEPC; ++j) acc_a[j] = 0.f;
+  if (nk > 0) {
+    const float scale = rsqrtf((float)DH);
+    for (int kb = 0; kb < nk; kb += ASTEP) {
+      float sc[NI];
+      float mt = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        float kf[KEPC];
+        kvrow<TKV>::get(kr[i], kf);
+        float d = 0.f;
+#pragma unroll
+        for (int j = 0; j < KEPC; ++j) d = fmaf(kf[j], qv[j], d);
+#pragma unroll
+        for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o);
+        const int kk = kb + (i * 16 + wave) * KPL + sub;
+        sc[i] = kk < nk ? d * scale : -INFINITY;
+        mt = fmaxf(mt, sc[i]);
+      }
+#pragma unroll
+      for (int o = 32; o >= LPK; o >>= 1) mt = fmaxf(mt, __shfl_xor(mt, o));
+      const float m_new = fmaxf(m_run, mt);
+      float pr[NI];
+      if (m_new != -INFINITY) {                               // else this wavefront has had no key yet
+        const float alpha = __expf(m_run - m_new);
+        l_run *= alpha;
+#pragma unroll
+        for (int j = 0; j < KEPC; ++j) acc_a[j] *= alpha;
+        m_run = m_new;
+      }
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        pr[i] = (m_new != -INFINITY) ? __expf(sc[i] - m_new) : 0.f;
+        l_run += pr[i];
+        float vf[KEPC];
+        kvrow<TKV>::get(vr[i], vf);
+#pragma unroll
+        for (int j = 0; j < KEPC; ++j) acc_a[j] = fmaf(pr[i], vf[j], acc_a[j]);
+      }
+      if (kb + ASTEP < nk) att_request(kb + ASTEP);
+    }
+  }
+  if (has_att) {
+    // key subgroups of a wavefront, then the sixteen wavefronts
+#pragma unroll
+    for (int o = 32; o >= LPK; o >>= 1) {
+      l_run += __shfl_xor(l_run, o);
+#pragma unroll
+      for (int j = 0; j < KEPC; ++j) acc_a[j] += __shfl_xor(acc_a[j], o);
+    }
+    if (lane < LPK) {
+#pragma unroll
+      for (int j = 0; j < KEPC; ++j) part[wave][el + j] = acc_a[j];
+    }
+    if (lane == 0) { stat[wave][0] = m_run; stat[wave][1] = l_run; }
+  }
+  __syncthreads();                                            // x in LDS; attention pieces in LDS
+  if (has_att) {
+    float mm = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mm = fmaxf(mm, stat[i][0]);
+    float* wout = oa.work + OA_HEAD + (int64_t)blockIdx.x * oa_pstride(DH);
+    for (int e = tid; e < DH + 2; e += 1024) {
+      float v = 0.f;
+      if (e < DH) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v += (stat[i][0] == -INFINITY ? 0.f : __expf(stat[i][0] - mm)) * part[i][e];
+      } else if (e == DH) {
+        v = mm;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v += (stat[i][0] == -INFINITY ? 0.f : __expf(stat[i][0] - mm)) * stat[i][1];
+      }
+      const int at = e < DH ? MTJ_DEC_PAD + e : e - DH;        // {max, sum, -, -, V[DH]}
+      __hip_atomic_store(wout + at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  // Every store of this workgroup has reached the coherence point before its arrival is counted.  The second weight
+  // tile is requested first: memory operations complete in order, so waiting until only its 8 loads are outstanding
+  // waits for the stores without waiting for the tile.
+  __builtin_amdgcn_sched_barrier(0);
+  if (n1 > 1) {
+    request(w2, 1, ta, tpr - ta);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0x0f78);                        // vmcnt(8), expcnt and lgkmcnt unconstrained
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0f70);                        // vmcnt(0)
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  __syncthreads();
+  // the value the counter had is not needed before the wait: nothing stalls on the atomic's return here
+  unsigned long long arrived_at = 0;
+  if (tid == 0)
+    arrived_at = __hip_atomic_fetch_add(reinterpret_cast<unsigned long long*>(oa.work), 1ull, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+
+  // ---- first pass: the columns that do not depend on the attention
+  float mine = 0.f, acc = 0.f;
+  int ct = ta, cr = 0;                                         // consumer cursor: tile, row
+  auto consume = [&](const uint32x4 (&t)[U], int t_end, bool add) {
+    const float* xk = xs + ct * TILE + lane * EPC;
+#pragma unroll
+    for (int u = 0; u < U; ++u) chunk<T>::fma(t[u], xk + u * STEP, acc);
+    if (++ct == t_end) {
+      const float sum = wave_sum(acc);
+      if (lane == cr) mine = add ? mine + sum : sum;
+      acc = 0.f; ++cr;
+      ct = add ? 0 : ta;
+    }
+  };
+  {
+    int g = 0;
+    for (; g + 3 < n1; g += 2) {                               // tiles g and g+1 are in w and w2
+      consume(w, tpr, false);
+      request(w, g + 2, ta, tpr - ta);
+      consume(w2, tpr, false);
+      request(w2, g + 3, ta, tpr - ta);
+    }
+    if (g + 2 < n1) {                                          // three left
+      consume(w, tpr, false);
+      request(w, g + 2, ta, tpr - ta);
+      consume(w2, tpr, false);
+      consume(w, tpr, false);
+    } else if (g + 1 < n1) {
+      consume(w, tpr, false);
+      consume(w2, tpr, false);
+    } else if (g < n1) {
+      consume(w, tpr, false);
+    }
+  }
+  // ---- second pass: the attention columns.  Their first tile is requested before the wait.
+  if (n2 > 0) request(w, 0, 0, ta);
+  if (tid == 0) {
+    const unsigned long long* cnt = reinterpret_cast<const unsigned long long*>(oa.work);
+    const unsigned long long target = (arrived_at / (unsigned)nwg + 1) * (unsigned)nwg;
+    unsigned spins = 0;
+    while (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+      __builtin_amdgcn_s_sleep(8);
+      if (++spins > (1u << 24)) {                              // some workgroup never arrived: give up, flag it
+        reinterpret_cast<unsigned*>(oa.work)[2] = 1u;
+        break;
+      }
+    }
+  }
+  __syncthreads();
+  for (int k = tid * 4; k < dm; k += 4096) {
+    const int hh = k / DH, e = k - hh * DH;
+    *reinterpret_cast<floatx4*>(xs + k) =
+        mtj_merge_partials(oa.work + OA_HEAD + (int64_t)hh * S * oa_pstride(DH), S, oa_pstride(DH), e);
+  }
+  __syncthreads();
+  ct = 0; cr = 0;
+  for (int g = 0; g < n2; ++g) {
+    consume(w, ta, true);
+    if (g + 1 < n2) request(w, g + 1, 0, ta);
+  }
+  if (lane < nrows) reinterpret_cast<float*>(a.out)[row0 + lane] = mine + pre_add;
+}
+
 template <typename T>
 int dispatch(const gemv_args& a, hipStream_t s) {
   constexpr int U = 8;
@@ -327,3 +608,90 @@ extern "C" int mtj_gemv(const float* x, const float* ln_scale, const float* ln_o
   if (dtype == MTJ_F16) return dispatch<f16_t>(a, s);
   return mtj_fail(MTJ_EDTYPE, "mtj_gemv: dtype %d", dtype);
 }
+
+// ------------------------------------------------------------------------------------------------ fused out projection
+namespace {
+
+constexpr int OA_TILE_BYTES = 8 * 64 * 16;     // one tile of 8 wavefront loads
+
+struct outatt_plan {
+  int grid, S;
+};
+
+// The fused kernel needs whole tiles on both sides of the attention/rest boundary and every workgroup resident at once.
+bool outatt_plan_for(int64_t N, int64_t K, int dtype, int64_t H, int64_t dh, int kv_dtype, int64_t Tcap, outatt_plan* plan) {
+  if (dtype != MTJ_F32 && dtype != MTJ_BF16) return false;
+  if (kv_dtype != (dtype == MTJ_F32 ? MTJ_F32 : MTJ_F16) || (dh != 64 && dh != 256) || H <= 0 || N <= 0) return false;
+  const int64_t tile = OA_TILE_BYTES / mtj_elem_size(dtype), dm = H * dh;
+  if (K % tile || dm % tile || dm >= K || K * 4 + 24 * 1024 > 160 * 1024) return false;
+  int64_t grid = 256;
+  if (grid > (N + 15) / 16) grid = (N + 15) / 16;
+  if ((N + grid * 16 - 1) / (grid * 16) > 62) return false;
+  static std::atomic<int> cus[MTJ_MAX_DEVICES];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MTJ_MAX_DEVICES) return false;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return false;
+    cus[dev].store(n, std::memory_order_relaxed);
+  }
+  if (grid > n) return false;
+  int64_t S = grid / H;
+  if (S > MTJ_DEC_MAXS) S = MTJ_DEC_MAXS;
+  if (S > (Tcap + 15) / 16) S = (Tcap + 15) / 16;
+  if (S < 1) return false;
+  plan->grid = (int)grid;
+  plan->S = (int)S;
+  return true;
+}
+
+template <typename T, typename TKV, int DH>
+int launch_outatt(const outatt_args& oa, int grid, hipStream_t s) {
+  const size_t lds = (size_t)oa.g.K * sizeof(float);
+  static mtj_device_once once;
+  if (int rc = mtj_allow_lds(once, "mtj_gemv_attn", &gemv_outatt_kernel<T, TKV, DH>, 160 * 1024 - 24 * 1024)) return rc;
+  gemv_outatt_kernel<T, TKV, DH><<<(unsigned)grid, 1024, lds, s>>>(oa);
+  return mtj_check_launch("mtj_gemv_attn");
+}
+
+}  // namespace
+
+extern "C" int mtj_gemv_attn_supported(int64_t N, int64_t K, int dtype, int64_t H, int64_t dh, int kv_dtype, int64_t Tcap) {
+  outatt_plan plan;
+  return outatt_plan_for(N, K, dtype, H, dh, kv_dtype, Tcap, &plan) ? 1 : 0;
+}
+
+extern "C" int64_t mtj_gemv_attn_work_bytes(int64_t H, int64_t dh) {
+  if (H <= 0 || dh <= 0) return 0;
+  return (OA_HEAD + H * MTJ_DEC_MAXS * ((dh + MTJ_DEC_PAD + 31) / 32 * 32)) * (int64_t)sizeof(float);
+}
+
+extern "C" int mtj_gemv_attn(const float* x, const void* W, const float* bias, int64_t N, int64_t K, int dtype, float* out,
+                             const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t H,
+                             int64_t Tcap, int64_t dh, int kv_dtype, void* work, void* stream) {
+  MTJ_REQUIRE(x && W && out && q && k_cache && v_cache && pos && work, MTJ_EINVAL, "mtj_gemv_attn: null pointer");
+  MTJ_REQUIRE(out != x, MTJ_EINVAL, "mtj_gemv_attn: out must be distinct from x");
+  MTJ_REQUIRE(mtj_aligned16(x) && mtj_aligned16(W) && mtj_aligned16(q) && mtj_aligned16(k_cache) && mtj_aligned16(v_cache) &&
+                  (reinterpret_cast<uintptr_t>(work) & 127u) == 0,
+              MTJ_EALIGN, "mtj_gemv_attn: x, W, q and the caches must be 16-byte aligned, work 128-byte aligned");
+  outatt_plan plan;
+  MTJ_REQUIRE(Tcap > 0 && outatt_plan_for(N, K, dtype, H, dh, kv_dtype, Tcap, &plan), MTJ_ELIMIT,
+              "mtj_gemv_attn: shape N=%lld K=%lld H=%lld dh=%lld is not covered by the fused kernel (see "
+              "mtj_gemv_attn_supported); use mtj_attn_decode_partials + mtj_gemv",
+              (long long)N, (long long)K, (long long)H, (long long)dh);
+  outatt_args oa{};
+  oa.g.x = x; oa.g.W = W; oa.g.bias = bias; oa.g.N = N; oa.g.K = K; oa.g.epi = MTJ_EPI_RESID; oa.g.out = out;
+  oa.g.out_dtype = MTJ_F32;
+  oa.q = q; oa.kc = k_cache; oa.vc = v_cache; oa.pos = pos; oa.H = (int)H; oa.Tcap = (int)Tcap; oa.S = plan.S;
+  oa.work = reinterpret_cast<float*>(work);
+  hipStream_t s = (hipStream_t)stream;
+#define MTJ_OA(WD, TW, KD, TK, DHV) \
+  if (dtype == WD && kv_dtype == KD && dh == DHV) return launch_outatt<TW, TK, DHV>(oa, plan.grid, s);
+  MTJ_OA(MTJ_BF16, bf16_t, MTJ_F16, f16_t, 256)
+  MTJ_OA(MTJ_BF16, bf16_t, MTJ_F16, f16_t, 64)
+  MTJ_OA(MTJ_F32, float, MTJ_F32, float, 256)
+  MTJ_OA(MTJ_F32, float, MTJ_F32, float, 64)
+#undef MTJ_OA
+  return mtj_fail(MTJ_ELIMIT, "mtj_gemv_attn: no kernel for weight dtype %d with K/V dtype %d", dtype, kv_dtype);
+}
+

@@ -53,6 +53,9 @@ SIGNATURES = {
     "mtj_gemm_splitk_ln": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _p, _i64, _p, _i64, _p, _p, _p, _i64, _i32,
                                  C.c_float, _p]),
     "mtj_gemv": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p, _i32, C.POINTER(InProj), C.POINTER(AttnMerge), _p]),
+    "mtj_gemv_attn_supported": (_i32, [_i64, _i64, _i32, _i64, _i64, _i32, _i64]),
+    "mtj_gemv_attn_work_bytes": (_i64, [_i64, _i64]),
+    "mtj_gemv_attn": (_i32, [_p, _p, _p, _i64, _i64, _i32, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i32, _p, _p]),
     "mtj_attn_prefill": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _p, _i64, _i32, _p, _p]),
     "mtj_attn_decode_splits": (_i32, [_i64, _i64, _i64]),
     "mtj_attn_decode_work_bytes": (_i64, [_i64, _i64, _i64, _i64]),

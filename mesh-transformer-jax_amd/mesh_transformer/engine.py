@@ -197,6 +197,11 @@ class Session:
         nb = max(nb, splitk_work_bound(M, d, d + F, w.mm_dtype))
         self.gemm_work = torch.empty(max(nb, 256), dtype=torch.uint8, device=dev)
         self.attn_work = torch.zeros(max(L.mtj_attn_decode_work_bytes(B, H, dh, Tcap), 256), dtype=torch.uint8, device=dev)
+        # batch 1: the out projection computes the attention itself when the shape allows it (its counter block is
+        # zeroed here, once, and then only the kernel touches it)
+        self.fused_attn = bool(self.gemv_path and cfg.get("fused_decode_attention", True) and
+                               L.mtj_gemv_attn_supported(d, d + F, w.dtype, H, dh, w.act_dtype, Tcap))
+        self.oa_work = torch.zeros(L.mtj_gemv_attn_work_bytes(H, dh), dtype=torch.uint8, device=dev) if self.fused_attn else None
         self.sample_work = None
         self.tok = torch.zeros(B, dtype=torch.int32, device=dev)
         self.pos = torch.zeros(B, dtype=torch.int32, device=dev)
@@ -323,6 +328,11 @@ class Engine:
             ip = self._inproj(ses, i, 1, ses.pos, ses.q, F32, ses.act, F32, None)
             check(L.mtj_gemv(ptr(ses.x), ptr(w.ln_s[i]), ptr(w.ln_o[i]), ptr(w.w_in[i]), ptr(w.b1[i]), 3 * d + F, d,
                              w.dtype, EPI_INPROJ, None, 0, C.byref(ip), None, s))
+            if ses.fused_attn:
+                check(L.mtj_gemv_attn(ptr(ses.act), ptr(w.w_out[i]), ptr(w.b2[i]), d, d + F, w.dtype, ptr(ses.x), ptr(ses.q),
+                                      ptr(ses.kc[i]), ptr(ses.vc[i]), ptr(ses.pos), self.H, ses.Tcap, self.dh, w.act_dtype,
+                                      ptr(ses.oa_work), s))
+                return
             # the per-range attention partials are merged by the out projection while it stages its input
             am = AttnMerge()
             check(L.mtj_attn_decode_partials(ptr(ses.q), ptr(ses.kc[i]), ptr(ses.vc[i]), ptr(ses.pos), B, self.H, ses.Tcap,

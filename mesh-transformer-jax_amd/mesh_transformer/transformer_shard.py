@@ -60,7 +60,8 @@ class CausalTransformer:
 
     config keys read: layers, d_model, n_heads, n_vocab, norm, pe, pe_rotary_dims, cores_per_replica,
     sampler (callable, transformer_shard.py:191), early_cast.  Extra, optional: "device",
-    "steps_per_graph" (decode steps recorded into one HIP graph, default 8; 0 disables graphs)."""
+    "steps_per_graph" (decode steps recorded into one HIP graph, default 8; 0 disables graphs),
+    "fused_decode_attention" (batch-1 decode computes the attention inside the out-projection launch, default True)."""
 
     def __init__(self, config, params=None):
         self.config = config
@@ -184,6 +185,9 @@ class CausalTransformer:
                 timing.update(prefill_s=t1 - t0, prefill_tokens=B * Tp, warmup_s=t2 - t1, decode_s=t3 - t2,
                               decode_steps=G - W)
             torch.cuda.synchronize(dev)
+            if ses.oa_work is not None and int(ses.oa_work[8:12].view(torch.int32)[0]) != 0:
+                raise RuntimeError("a fused out-projection launch gave up waiting for its attention partials; "
+                                   "set config['fused_decode_attention'] = False")
             toks = ses.out_tokens[:, :G].cpu().numpy().astype(np.uint32)[:, :, None]
             final_state = (toks[:, -1], ses, None)
             out = (toks, None)

@@ -589,6 +589,53 @@ def test_attn_decode_partials_merged_by_the_out_projection_gemv(L, dt, dh, H, F,
     assert rel_err(x, ref) < 5e-6, (dt, dh, Tcap, p)
 
 
+@pytest.mark.parametrize("dt,dh,H,F", [("f16", 256, 16, 16384), ("f32", 64, 32, 8192), ("f16", 64, 64, 4096)])
+def test_out_projection_with_the_attention_inside(L, dt, dh, H, F):
+    """mtj_gemv_attn: x += [attention(q, window) | gelu] @ W_out + b in ONE launch (the attention partials are produced
+    by the first workgroups and merged behind an arrival counter), against the float64 evaluation of
+    layers.py:275-285, 290, 313 - several window fills, launches back to back on one counter block."""
+    a = abi()
+    wdt = "f32" if dt == "f32" else "bf16"
+    d = H * dh
+    Tcap = 2047
+    assert L.mtj_gemv_attn_supported(d, d + F, a.dtype_code(TD[wdt]), H, dh, a.dtype_code(TD[dt]), Tcap) == 1
+    g = torch.Generator().manual_seed(dh + H)
+    kc = torch.randn(1, H, Tcap, dh, generator=g).to(TD[dt]).to(DEV)
+    vc = torch.randn(1, H, Tcap, dh, generator=g).to(TD[dt]).to(DEV)
+    Wh = (torch.randn(d + F, d, generator=g) * 0.02).to(TD[wdt]).to(DEV)
+    W = _packed(Wh)
+    bias = torch.randn(d, generator=g).to(DEV)
+    work = torch.zeros(L.mtj_gemv_attn_work_bytes(H, dh), dtype=torch.uint8, device=DEV)
+    for p in (650, 0, 5, 2046, 7000, 63):
+        q = torch.randn(1, H, dh, generator=g).to(DEV)
+        act = torch.randn(1, d + F, generator=g).to(DEV)
+        act[:, :d] = float("nan")                              # the attention columns must not be read from x
+        x0 = torch.randn(d, generator=g).to(DEV)
+        x = x0.clone()
+        pos = torch.tensor([p], dtype=torch.int32, device=DEV)
+        a.check(L.mtj_gemv_attn(a.ptr(act), a.ptr(W), a.ptr(bias), d, d + F, a.dtype_code(TD[wdt]), a.ptr(x), a.ptr(q),
+                                a.ptr(kc), a.ptr(vc), a.ptr(pos), H, Tcap, dh, a.dtype_code(TD[dt]), a.ptr(work), S()))
+        torch.cuda.synchronize()
+        n = min(p + 1, Tcap)
+        sc = torch.einsum("hd,hTd->hT", q[0].double(), kc[0, :, :n].double()) / math.sqrt(dh)
+        att = torch.einsum("hT,hTd->hd", torch.softmax(sc, -1), vc[0, :, :n].double()).reshape(-1)
+        ref = x0.double() + torch.cat([att, act[0, d:].double()]) @ Wh.double() + bias.double()
+        assert rel_err(x, ref) < 5e-6, (dt, dh, p)
+    words = work[:16].view(torch.int32).cpu()
+    assert int(words[2]) == 0                                  # no launch gave up waiting
+    assert int(words[0]) % 6 == 0 and int(words[0]) > 0        # six launches, every workgroup arrived each time
+
+
+def test_out_projection_with_attention_refuses_other_shapes(L):
+    a = abi()
+    assert L.mtj_gemv_attn_supported(512, 2560, a.BF16, 8, 64, a.F16, 200) == 0     # K is not a whole number of tiles
+    assert L.mtj_gemv_attn_supported(4096, 4096, a.BF16, 16, 256, a.F16, 200) == 0  # nothing but attention columns
+    t = torch.zeros(4096, device=DEV)
+    rc = L.mtj_gemv_attn(a.ptr(t), a.ptr(t), None, 512, 2560, a.BF16, a.ptr(t[2048:]), a.ptr(t), a.ptr(t), a.ptr(t),
+                         a.ptr(t.view(torch.int32)), 8, 200, 64, a.F16, a.ptr(t), S())
+    assert rc == -5 and b"mtj_gemv_attn_supported" in L.mtj_last_error()
+
+
 # ------------------------------------------------------------------ the same kernels as torch.ops.mtj operators
 def test_torch_ops_reach_the_same_kernels():
     from mesh_transformer import ops  # noqa: F401

@@ -153,6 +153,18 @@ int mtj_gemm_splitk_ln(const void* A, int64_t lda, const void* W, const float* b
                        int dtype, float* x, int64_t ldx, void* work, int64_t work_bytes, const float* ln_scale,
                        const float* ln_offset, void* h, int64_t ldh, int h_dtype, float alpha, void* stream);
 
+/* ProjectionShard.loss (layers.py:569-593) without the logits ever reaching memory: the rows of A are the
+ * LayerNorm'd activations, logits = alpha * A x W^T + bias are formed tile by tile on the matrix cores and reduced in
+ * the epilogue to (maximum, sum of exp(logit - maximum), logit of the target column) per row and column tile; a
+ * second, tiny launch merges the tiles: loss[m] = log(sum exp(l - max)) - (l[target] - max), correct[m] =
+ * (l[target] == max), exactly what mtj_xent computes from stored logits (a target outside [0, N) selects nothing).
+ * `work`: mtj_gemm_xent_work_bytes(M, N, dtype) bytes (2 floats per row and column tile + 1 per row, against
+ * 4 * N bytes per row for the logits themselves); correct may be NULL. */
+int64_t mtj_gemm_xent_work_bytes(int64_t M, int64_t N, int dtype);
+int mtj_gemm_xent(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
+                  int dtype, float alpha, const int32_t* target, float* loss, uint8_t* correct, void* work,
+                  int64_t work_bytes, void* stream);
+
 /* Batch-1 decode matrix-vector product: y = f(x) @ W^T with float32 activations and float32 accumulation
  * (jnp.dot(f32, bf16) semantics of hk.Linear at decode, layers.py:316-344).  x float32 [K].
  * If ln_scale != NULL the kernel first applies LayerNorm(x) (layers.py:17-36) - x then has K = d entries.

@@ -69,7 +69,14 @@ struct gemm_args {
   int splits;             // > 1: blockIdx.y owns a K range and stores a raw float32 partial at out + y * split_stride
   int64_t split_stride;
   mtj_inproj ip;
+  // MTJ_EPI_XENT: the product is never stored; per (row, column tile) the maximum and the sum of exp(logit - maximum)
+  const int32_t* target;  // [M]
+  float* pmax;            // [tiles_n, M]
+  float* psum;            // [tiles_n, M]
+  float* tlogit;          // [M]: the logit of the target column (written by the one tile that holds it)
 };
+
+constexpr int MTJ_EPI_XENT = 3;   // internal: logits + cross entropy (ProjectionShard.loss, layers.py:569-593)
 
 // 16 consecutive elements, 16-byte vector stores (idx is a multiple of 16 elements, base 16-byte aligned)
 __device__ __forceinline__ void store16(void* base, int64_t idx, const float* v, int dtype) {
@@ -116,7 +123,72 @@ __device__ __forceinline__ void epilogue(const gemm_args& a, void* out, floatx16
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int fr = lane & 31, fg = lane >> 5;
-  if (EPI == MTJ_EPI_INPROJ) {
+  if (EPI == MTJ_EPI_XENT) {
+    // Row statistics of this workgroup's column tile: accumulator register v of lane (fr, fg) is row 8*(v/4) + 4*fg +
+    // v%4, column fr of a 32x32 tile, so a row is reduced over the WN tiles in registers, then over the 32 lanes
+    // with the same fg by shuffles, then over the WAVES_N wavefronts through LDS.
+    constexpr int BN = WAVES_N * WN * 32;
+    __syncthreads();                                       // every wavefront is done with the operand tiles
+    float* red = reinterpret_cast<float*>(smem);           // [WAVES_N][BM][2]
+    for_tiles<0, 0, WM, 1>([&](auto I_, auto) {
+      constexpr int i = decltype(I_)::value;
+      float val[WN][16];
+      int col[WN];
+      for_tiles<0, 0, 1, WN>([&](auto, auto J_) {
+        constexpr int j = decltype(J_)::value;
+        const int n = n0 + (wn * WN + j) * 32 + fr;
+        col[j] = n;
+        const bool n_ok = n < a.N;
+        const float bias = (a.bias && n_ok) ? a.bias[n] : 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) val[j][v] = n_ok ? acc[i][j][v] * a.alpha + bias : -INFINITY;
+      });
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int r = (wm * WM + i) * 32 + 8 * (v / 4) + 4 * fg + (v % 4);
+        const int m = m0 + r;
+        float mx = val[0][v];
+#pragma unroll
+        for (int j = 1; j < WN; ++j) mx = fmaxf(mx, val[j][v]);
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        float sm = 0.f;
+        if (mx != -INFINITY) {
+#pragma unroll
+          for (int j = 0; j < WN; ++j) sm += __expf(val[j][v] - mx);      // exp(-inf) = 0 for columns beyond N
+        }
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) sm += __shfl_xor(sm, o);
+        if (m < a.M) {
+          const int t = a.target[m];
+#pragma unroll
+          for (int j = 0; j < WN; ++j)
+            if (col[j] == t) a.tlogit[m] = val[j][v];
+        }
+        if (fr == 0) {
+          red[(wn * BM + r) * 2] = mx;
+          red[(wn * BM + r) * 2 + 1] = sm;
+        }
+      }
+    });
+    __syncthreads();
+    const int tn = n0 / BN;
+    for (int r = tid; r < BM; r += NT) {
+      const int m = m0 + r;
+      if (m >= a.M) continue;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < WAVES_N; ++w) mx = fmaxf(mx, red[(w * BM + r) * 2]);
+      float sm = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES_N; ++w) {
+        const float pm = red[(w * BM + r) * 2];
+        sm += pm == -INFINITY ? 0.f : __expf(pm - mx) * red[(w * BM + r) * 2 + 1];
+      }
+      a.pmax[(int64_t)tn * a.M + m] = mx;
+      a.psum[(int64_t)tn * a.M + m] = sm;
+    }
+  } else if (EPI == MTJ_EPI_INPROJ) {
     // Each 32x32 accumulator tile goes through a private LDS patch of its wavefront and comes back with one
     // lane owning 16 consecutive columns of one row: rotary pairs are then lane-local and every destination
     // (q, K/V window, gelu(fc_in)) gets 32- or 64-byte stores.
@@ -577,6 +649,7 @@ template <typename T, int BK>
 int dispatch(const gemm_args& a, int epi, hipStream_t s) {
   if (epi == MTJ_EPI_STORE) return dispatch_tile<T, MTJ_EPI_STORE, BK>(a, s);
   if (epi == MTJ_EPI_RESID) return dispatch_tile<T, MTJ_EPI_RESID, BK>(a, s);
+  if (epi == MTJ_EPI_XENT) return dispatch_tile<T, MTJ_EPI_XENT, BK>(a, s);
   return dispatch_tile<T, MTJ_EPI_INPROJ, BK>(a, s);
 }
 
@@ -692,6 +765,31 @@ __global__ __launch_bounds__(1024) void splitk_reduce_ln_kernel(const float* __r
       }
     }
   }
+}
+
+// Second half of the fused logits + cross entropy: merges the per-column-tile statistics of a row.
+// loss = log(sum exp(l - max)) - (l[target] - max), correct = (l[target] == max); a target outside [0, N) selects
+// nothing (pred = 0), as in xent_kernel.
+__global__ __launch_bounds__(256) void xent_merge_kernel(const float* __restrict__ pmax, const float* __restrict__ psum,
+                                                         const float* __restrict__ tlogit, const int32_t* __restrict__ target,
+                                                         int M, int N, int tiles_n, float* __restrict__ loss,
+                                                         uint8_t* __restrict__ correct) {
+  const int m = blockIdx.x * blockDim.x + threadIdx.x;
+  if (m >= M) return;
+  float mx = -INFINITY;
+  for (int t = 0; t < tiles_n; ++t) mx = fmaxf(mx, pmax[(int64_t)t * M + m]);
+  float sm = 0.f;
+  for (int t = 0; t < tiles_n; ++t) sm += __expf(pmax[(int64_t)t * M + m] - mx) * psum[(int64_t)t * M + m];
+  const int tg = target[m];
+  const float pred = ((uint32_t)tg < (uint32_t)N) ? tlogit[m] - mx : 0.f;
+  loss[m] = logf(sm) - pred;
+  if (correct) correct[m] = (pred == 0.f) ? 1 : 0;
+}
+
+// column-tile width that dispatch_tile will use for this problem
+int xent_tile_n(int64_t M, int64_t N, int dtype) {
+  if (M > 64 && dtype != MTJ_F32 && ((M + 255) / 256) * ((N + 255) / 256) >= 200) return 256;
+  return 128;
 }
 
 // how many K ranges a skinny problem is cut into so that its few output tiles still fill the chip
@@ -834,4 +932,33 @@ extern "C" int mtj_gemm_splitk_ln(const void* A, int64_t lda, const void* W, con
   splitk_reduce_ln_kernel<<<(unsigned)M, 1024, 0, s>>>((const float*)work, splits, M * N, (int)N, bias, x, ldx, ln_scale,
                                                        ln_offset, h, ldh, h_dtype);
   return mtj_check_launch("mtj_gemm_splitk_ln");
+}
+
+extern "C" int64_t mtj_gemm_xent_work_bytes(int64_t M, int64_t N, int dtype) {
+  if (M <= 0 || N <= 0 || !mtj_is_dtype(dtype)) return 0;
+  const int64_t tiles_n = (N + xent_tile_n(M, N, dtype) - 1) / xent_tile_n(M, N, dtype);
+  return (2 * tiles_n + 1) * M * (int64_t)sizeof(float);
+}
+
+extern "C" int mtj_gemm_xent(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
+                             int dtype, float alpha, const int32_t* target, float* loss, uint8_t* correct, void* work,
+                             int64_t work_bytes, void* stream) {
+  if (int rc = check_common(A, lda, W, M, N, K, dtype, "mtj_gemm_xent")) return rc;
+  MTJ_REQUIRE(target && loss && work, MTJ_EINVAL, "mtj_gemm_xent: null pointer");
+  MTJ_REQUIRE(mtj_aligned16(work) && work_bytes >= mtj_gemm_xent_work_bytes(M, N, dtype), MTJ_EINVAL,
+              "mtj_gemm_xent: work must hold mtj_gemm_xent_work_bytes() bytes");
+  const int bn = xent_tile_n(M, N, dtype);
+  const int64_t tiles_n = (N + bn - 1) / bn;
+  gemm_args a{};
+  a.A = A; a.lda = lda; a.W = W; a.bias = bias; a.M = (int)M; a.N = (int)N; a.K = (int)K;
+  a.alpha = alpha; a.splits = 1;
+  a.target = target;
+  a.pmax = reinterpret_cast<float*>(work);
+  a.psum = a.pmax + tiles_n * M;
+  a.tlogit = a.psum + tiles_n * M;
+  hipStream_t s = (hipStream_t)stream;
+  if (int rc = dispatch_dtype(a, dtype, MTJ_EPI_XENT, s)) return rc;
+  xent_merge_kernel<<<(unsigned)((M + 255) / 256), 256, 0, s>>>(a.pmax, a.psum, a.tlogit, target, (int)M, (int)N, (int)tiles_n,
+                                                              loss, correct);
+  return mtj_check_launch("mtj_gemm_xent");
 }

@@ -52,6 +52,8 @@ SIGNATURES = {
     "mtj_gemm_splitk": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, _p, _i64, C.c_float, _p]),
     "mtj_gemm_splitk_ln": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _p, _i64, _p, _i64, _p, _p, _p, _i64, _i32,
                                  C.c_float, _p]),
+    "mtj_gemm_xent_work_bytes": (_i64, [_i64, _i64, _i32]),
+    "mtj_gemm_xent": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, C.c_float, _p, _p, _p, _p, _i64, _p]),
     "mtj_gemv": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p, _i32, C.POINTER(InProj), C.POINTER(AttnMerge), _p]),
     "mtj_gemv_attn_supported": (_i32, [_i64, _i64, _i32, _i64, _i64, _i32, _i64]),
     "mtj_gemv_attn_work_bytes": (_i64, [_i64, _i64]),

@@ -266,6 +266,20 @@ class Engine:
         check(L.mtj_gemm(ptr(h), d, ptr(w.w_p_mm), ptr(w.b_p), M, V, d, w.mm_dtype, EPI_STORE, ptr(out), V, F32, None,
                          w.alpha_p, s))
 
+    def project_loss(self, ses, x, target, loss, correct):
+        """ProjectionShard.loss (layers.py:569-593) on every row of x against target [M] int32: loss [M] float32 and
+        correct [M] uint8.  The logits live only in the accumulators of the projection GEMM, whose epilogue keeps
+        (max, sum of exp, target logit) per row and column tile."""
+        L, w, s = _abi.lib(), self.w, _abi.stream_handle()
+        M, d, V = x.shape[0], w.d, w.V
+        h = ses.h_pf[:M]
+        need = L.mtj_gemm_xent_work_bytes(M, V, w.mm_dtype)
+        if getattr(ses, "xent_work", None) is None or ses.xent_work.numel() * 4 < need:
+            ses.xent_work = torch.empty((need + 3) // 4, dtype=torch.float32, device=x.device)
+        check(L.mtj_layernorm(ptr(x), ptr(w.pln_s), ptr(w.pln_o), M, d, ptr(h), w.act_dtype, s))
+        check(L.mtj_gemm_xent(ptr(h), d, ptr(w.w_p_mm), ptr(w.b_p), M, V, d, w.mm_dtype, w.alpha_p, ptr(target),
+                              ptr(loss), ptr(correct), ptr(ses.xent_work), ses.xent_work.numel() * 4, s))
+
     def layer_prefill(self, ses, i, x, h, act, Tp, pos0, key_limit=None):
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()
         M, d, F = x.shape[0], w.d, w.F

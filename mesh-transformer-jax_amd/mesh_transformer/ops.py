@@ -18,6 +18,7 @@ hop per launch would buy nothing).  Operators that write into caller-owned memor
     torch.ops.mtj.attn_prefill(q, k_cache, v_t, pos0, Tp, key_limit)   self_attn + masks        layers.py:260-285,347-366
     torch.ops.mtj.attn_decode(q, k_cache, v_cache, pos, out_dtype) one-token attention          layers.py:316-344
     torch.ops.mtj.xent(logits, target)                             ProjectionShard.loss         layers.py:569-593
+    torch.ops.mtj.gemm_xent(A, W, bias, alpha, target)             ... on logits never stored   layers.py:559,569-593
     torch.ops.mtj.sample_greedy(logits) / sample_nucleus(...)      config["sampler"]            sampling.py:6-44
 """
 import ctypes as C
@@ -95,6 +96,20 @@ def _gemm(A, W, bias, alpha, out_dtype):
     check(_abi.lib().mtj_gemm(ptr(A), A.stride(0), ptr(W), ptr(bias), M, N, K, _code(W), EPI_STORE, ptr(out), N, out_dtype,
                               None, alpha, _s()))
     return out
+
+
+def _gemm_xent(A, W, bias, alpha, target):
+    M, K = A.shape
+    N = W.shape[0]
+    L = _abi.lib()
+    nb = L.mtj_gemm_xent_work_bytes(M, N, _code(W))
+    work = torch.empty(nb, dtype=torch.uint8, device=A.device)
+    loss = torch.empty(M, dtype=torch.float32, device=A.device)
+    correct = torch.empty(M, dtype=torch.uint8, device=A.device)
+    target = target.reshape(-1).to(torch.int32).contiguous()
+    check(L.mtj_gemm_xent(ptr(A), A.stride(0), ptr(W), ptr(bias), M, N, K, _code(W), alpha, ptr(target), ptr(loss),
+                          ptr(correct), ptr(work), nb, _s()))
+    return loss, correct.bool()
 
 
 def _gemm_resid_(x, A, W, bias, alpha):
@@ -189,6 +204,7 @@ _define("xent(Tensor logits, Tensor target) -> (Tensor, Tensor)", _xent)
 _define("pack_weight(Tensor w) -> Tensor", _pack_weight)
 _define("pack_weight_f16(Tensor w, float scale) -> Tensor", _pack_weight_f16)
 _define("gemm(Tensor A, Tensor W, Tensor? bias, float alpha, int out_dtype) -> Tensor", _gemm)
+_define("gemm_xent(Tensor A, Tensor W, Tensor? bias, float alpha, Tensor target) -> (Tensor, Tensor)", _gemm_xent)
 _define("gemm_resid_(Tensor(a!) x, Tensor A, Tensor W, Tensor? bias, float alpha) -> ()", _gemm_resid_)
 _define("gemv(Tensor x, Tensor W, Tensor? bias, Tensor? ln_scale, Tensor? ln_offset) -> Tensor", _gemv)
 _define("inproj_(Tensor h, Tensor W, Tensor b1, float alpha, Tensor pos0, Tensor sin_tab, Tensor cos_tab, Tensor(a!) q, "
@@ -200,5 +216,5 @@ _define("sample_greedy(Tensor logits) -> Tensor", _sample_greedy)
 _define("sample_nucleus(Tensor logits, Tensor top_p, Tensor temp, Tensor? top_k, Tensor uniforms) -> (Tensor, Tensor, Tensor)",
         _sample_nucleus)
 
-OPS = ("layernorm", "embed", "xent", "pack_weight", "pack_weight_f16", "gemm", "gemm_resid_", "gemv", "inproj_",
+OPS = ("layernorm", "embed", "xent", "pack_weight", "pack_weight_f16", "gemm", "gemm_xent", "gemm_resid_", "gemv", "inproj_",
        "attn_prefill", "attn_decode", "sample_greedy", "sample_nucleus")

@@ -259,14 +259,7 @@ class CausalTransformer:
             x = eng.prefill(ses, rect, T, key_limit=limit)
             loss = torch.empty(B * T, dtype=torch.float32, device=dev)
             correct = torch.empty(B * T, dtype=torch.uint8, device=dev)
-            # the logits of a slab of rows at a time: [B*T, V] float32 need not exist all at once
-            rows = max(1, min(B * T, (1 << 30) // (4 * V)))
-            logits = torch.empty(rows, V, dtype=torch.float32, device=dev)
-            for r0 in range(0, B * T, rows):
-                n = min(rows, B * T - r0)
-                eng.project(ses, x[r0:r0 + n], logits[:n])
-                _abi.check(L.mtj_xent(_abi.ptr(logits), V, _abi.ptr(target[r0:r0 + n]), n, V, _abi.ptr(loss[r0:r0 + n]),
-                                      _abi.ptr(correct[r0:r0 + n]), _abi.stream_handle()))
+            eng.project_loss(ses, x, target, loss, correct)       # the [B*T, V] logits are never stored
             torch.cuda.synchronize(dev)
             all_loss = loss.view(B, T).cpu().numpy()
             return {"loss": all_loss.mean(-1), "last_loss": all_loss[:, -1].copy(), "all_loss": all_loss,

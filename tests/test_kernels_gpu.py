@@ -778,6 +778,49 @@ def test_xent_rows(L, M, V, ld):
     assert torch.equal(correct.bool(), want)
 
 
+@pytest.mark.parametrize("dt,M,V,K", [("f32", 37, 50400, 256), ("bf16", 37, 50400, 512), ("f16", 64, 1000, 256),
+                                      ("f32", 200, 1000, 256), ("bf16", 300, 5000, 128), ("f16", 1, 132, 64),
+                                      ("bf16", 2048, 50400, 1024), ("f16", 2000, 50400, 512)])
+def test_logits_and_cross_entropy_in_one_gemm(L, dt, M, V, K):
+    """mtj_gemm_xent against mtj_gemm (STORE) + mtj_xent on the same operands and against float64; the last two shapes
+    are 8 x 197 tiles of 256 x 256 (the direct-to-LDS kernel, ragged in both directions), the others the 32-, 64- and
+    128-row tiles.  Targets include the row's best column, a column in the ragged last tile and one outside the vocabulary."""
+    a = abi()
+    g = torch.Generator().manual_seed(M + V + K)
+    A = torch.randn(M, K, generator=g).to(TD[dt]).to(DEV)
+    Wh = (torch.randn(K, V, generator=g) * 0.2).to(TD[dt]).to(DEV)
+    bias = torch.randn(V, generator=g).to(DEV)
+    W = _packed(Wh)
+    code, alpha = a.dtype_code(TD[dt]), 0.5
+    logits = torch.empty(M, V, device=DEV)
+    a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, V, K, code, a.EPI_STORE, a.ptr(logits), V, 0, None, alpha, S()))
+    tgt = torch.randint(0, V, (M,), generator=g).to(torch.int32).to(DEV)
+    best = logits.argmax(-1).to(torch.int32)
+    tgt[::3] = best[::3]
+    if M > 4:
+        tgt[1] = V - 1
+        tgt[4] = V + 5
+    loss0, loss1 = torch.empty(M, device=DEV), torch.full((M,), -1.0, device=DEV)
+    ok0, ok1 = torch.empty(M, dtype=torch.uint8, device=DEV), torch.full((M,), 7, dtype=torch.uint8, device=DEV)
+    a.check(L.mtj_xent(a.ptr(logits), V, a.ptr(tgt), M, V, a.ptr(loss0), a.ptr(ok0), S()))
+    nb = L.mtj_gemm_xent_work_bytes(M, V, code)
+    assert 0 < nb <= (2 * ((V + 127) // 128) + 1) * M * 4
+    work = torch.full((nb // 4,), float("nan"), device=DEV)              # nothing is expected to be there
+    a.check(L.mtj_gemm_xent(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, V, K, code, alpha, a.ptr(tgt), a.ptr(loss1), a.ptr(ok1),
+                            a.ptr(work), nb, S()))
+    torch.cuda.synchronize()
+    assert torch.equal(ok1, ok0)
+    assert (loss1 - loss0).abs().max().item() < 2e-5 * max(1.0, loss0.abs().max().item())
+    l64 = alpha * (A.double() @ Wh.double()) + bias.double()
+    inside = tgt.long() < V
+    ref = torch.logsumexp(l64, -1) - torch.where(inside, l64.gather(1, tgt.long().clamp(max=V - 1)[:, None])[:, 0],
+                                                 l64.max(-1).values)
+    assert (loss1.double() - ref).abs().max().item() < 2e-5 * max(1.0, ref.abs().max().item())
+    with pytest.raises(ValueError):
+        a.check(L.mtj_gemm_xent(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, V, K, code, alpha, a.ptr(tgt), a.ptr(loss1),
+                                a.ptr(ok1), a.ptr(work), nb - 4, S()))
+
+
 def test_greedy_lowest_index_on_ties(L):
     a = abi()
     V = 50400

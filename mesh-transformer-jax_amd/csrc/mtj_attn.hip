@@ -38,14 +38,11 @@ template <> struct mma<f16_t> {
     return f;
   }
   __device__ static __forceinline__ void pin(frag& f) { asm volatile("" : "+v"(f.v)); }
+  // 8 probabilities -> operand; they lie in [0, 64], so the conversion needs no clamp to the float16 range
   __device__ static __forceinline__ frag from_floats(const float* p) {
     frag f;
-    uint32x4 u;
-    u.x = pack_f16x2(p[0], p[1]);
-    u.y = pack_f16x2(p[2], p[3]);
-    u.z = pack_f16x2(p[4], p[5]);
-    u.w = pack_f16x2(p[6], p[7]);
-    f.v = *reinterpret_cast<f16x8*>(&u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f.v[j] = (f16_t)p[j];
     return f;
   }
   __device__ static __forceinline__ void run(floatx16& c, const frag& a, const frag& b) {
@@ -159,19 +156,29 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
   // Loads are unconditional: K rows beyond the last key are clamped to it (the causal mask removes them), and a
   // V^T row is ldvt >= round_up(Tp, BKV) long, so the chunk exists; what it holds beyond the last key is zeroed
   // in LDS by fix_last_tile (0 x garbage must not become NaN).
+  // Per-thread bases, so that a tile costs one scalar offset and no per-chunk address arithmetic: chunk i of the K
+  // tile is row i * (NT / CPRK) + tid / CPRK, chunk i of the V^T tile is row i * (NT / CPRV) + tid / CPRV.
+  static_assert(NT % CPRK == 0 && NT % CPRV == 0, "chunks of one pass start in the same column");
+  const int k_row0 = tid / CPRK;
+  const T* k_base = kc + bh * Tcap * DH + (tid % CPRK) * EPC;
+  const T* v_base = vt + (bh * DH + tid / CPRV) * ldvt + (tid % CPRV) * EPC;
+  const int64_t v_pass = (int64_t)(NT / CPRV) * ldvt;
   auto load_tile = [&](int kt) {
     const int key0 = kt * BKV;
+    if (key0 + BKV - 1 <= klast) {             // workgroup-uniform: every row of the tile exists
+      const T* kp = k_base + (int64_t)(key0 + k_row0) * DH;
 #pragma unroll
-    for (int i = 0; i < K_CHUNKS; ++i) {
-      const int c = i * NT + tid, row = c / CPRK, cc = c % CPRK;
-      const int key = (key0 + row <= klast) ? key0 + row : klast;
-      rk[i] = *reinterpret_cast<const uint32x4*>(kc + (bh * Tcap + key) * DH + cc * EPC);
-    }
+      for (int i = 0; i < K_CHUNKS; ++i) rk[i] = *reinterpret_cast<const uint32x4*>(kp + i * (NT / CPRK) * DH);
+    } else {
 #pragma unroll
-    for (int i = 0; i < V_CHUNKS; ++i) {
-      const int c = i * NT + tid, row = c / CPRV, cc = c % CPRV;
-      rv[i] = *reinterpret_cast<const uint32x4*>(vt + (bh * DH + row) * ldvt + key0 + cc * EPC);
+      for (int i = 0; i < K_CHUNKS; ++i) {
+        const int row = key0 + k_row0 + i * (NT / CPRK);
+        rk[i] = *reinterpret_cast<const uint32x4*>(k_base + (int64_t)(row <= klast ? row : klast) * DH);
+      }
     }
+    const T* vp = v_base + key0;
+#pragma unroll
+    for (int i = 0; i < V_CHUNKS; ++i) rv[i] = *reinterpret_cast<const uint32x4*>(vp + i * v_pass);
   };
   auto fix_last_tile = [&](int kt, int buf) {     // workgroup-uniform caller; runs between the store and the barrier
     const int key0 = kt * BKV;
@@ -180,17 +187,15 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
     raw_t* vs = reinterpret_cast<raw_t*>(Vs + buf * DH * VROW);
     for (int c = tid; c < DH * nbad; c += NT) vs[(c / nbad) * VROW + (BKV - nbad) + (c % nbad)] = (raw_t)0;
   };
+  T* ks_dst = Ks + k_row0 * KROW + (tid % CPRK) * EPC;
+  T* vs_dst = Vs + (tid / CPRV) * VROW + (tid % CPRV) * EPC;
   auto store_tile = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < K_CHUNKS; ++i) {
-      const int c = i * NT + tid, row = c / CPRK, cc = c % CPRK;
-      *reinterpret_cast<uint32x4*>(Ks + (buf * BKV + row) * KROW + cc * EPC) = rk[i];
-    }
+    for (int i = 0; i < K_CHUNKS; ++i)
+      *reinterpret_cast<uint32x4*>(ks_dst + (buf * BKV + i * (NT / CPRK)) * KROW) = rk[i];
 #pragma unroll
-    for (int i = 0; i < V_CHUNKS; ++i) {
-      const int c = i * NT + tid, row = c / CPRV, cc = c % CPRV;
-      *reinterpret_cast<uint32x4*>(Vs + (buf * DH + row) * VROW + cc * EPC) = rv[i];
-    }
+    for (int i = 0; i < V_CHUNKS; ++i)
+      *reinterpret_cast<uint32x4*>(vs_dst + (buf * DH + i * (NT / CPRV)) * VROW) = rv[i];
   };
 
   const int ntiles = (kmax >= 0) ? kmax / BKV + 1 : 0;
@@ -267,10 +272,16 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
         const float mnew = fmaxf(mrun, mt);
         const float alpha = (mnew == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(mrun - mnew);   // mrun = -inf -> 0
         lrun *= alpha;
+        // The accumulators live in the accumulation registers, which only the matrix instructions and copies can
+        // address; the empty asm statements tie each block to those registers on both sides of its multiplication,
+        // so that the copies out and back stay inside this rarely taken branch instead of the head of the key loop.
 #pragma unroll
-        for (int i = 0; i < NBLK; ++i)
+        for (int i = 0; i < NBLK; ++i) {
+          if constexpr (sizeof(T) == 2) asm volatile("" : "+a"(o[i]));
 #pragma unroll
           for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
+          if constexpr (sizeof(T) == 2) asm volatile("" : "+a"(o[i]));
+        }
         mrun = mnew;
       }
       const float msafe = (mrun == -INFINITY) ? 0.f : mrun;

@@ -60,6 +60,8 @@ enum {
  * Geometry and destinations of the fused input projection.  Row m of the GEMM is token t = m % Tp of
  * sequence b = m / Tp, at absolute position pos = pos0[b] + t; rows with pos < 0 are left padding and
  * write nothing to the cache.  Output columns: [0,d) q, [d,2d) v, [2d,3d) k, [3d,3d+F) fc_in.
+ * Precondition: every position is < max_pos.  A larger one is rotated with the LAST table row instead of reading
+ * beyond the tables (memory safe, numerically wrong), so the caller sizes the tables for prompt + generated tokens.
  */
 typedef struct {
   int32_t n_heads, d_head, rotary_dims; /* H, dh, r (r even, r <= dh)                                   */
@@ -70,7 +72,7 @@ typedef struct {
   const float* sin_tab;                 /* [max_pos, r/2] float32, rounded once from float64           */
   const float* cos_tab;                 /* [max_pos, r/2]                                              */
   void* q;                              /* [B, H, Tp, dh] in q_dtype                                   */
-  int32_t q_dtype;                      /* MTJ_F32 (decode attention reads float32 q) or MTJ_BF16      */
+  int32_t q_dtype;                      /* MTJ_F32 (decode attention reads float32 q) or a 16-bit type */
   int32_t kv_dtype;                     /* storage type of k_cache, v_cache and v_t                    */
   void* k_cache;                        /* [B, H, Tcap, dh] kv_dtype, rotated keys                     */
   void* v_cache;                        /* [B, H, Tcap, dh] kv_dtype                                   */

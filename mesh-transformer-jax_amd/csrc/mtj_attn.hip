@@ -512,7 +512,6 @@ int decode_splits(int64_t B, int64_t H, int64_t Tcap) {
   int64_t S = 256 / (B * H);
   if (S > (Tcap + 15) / 16) S = (Tcap + 15) / 16;
   if (S > MTJ_DEC_MAXS) S = MTJ_DEC_MAXS;
-  if (const char* e = getenv("MTJ_DEC_S")) { const int v = atoi(e); if (v >= 1 && v <= MTJ_DEC_MAXS && S > v) S = v; }
   if (S < 1) S = 1;
   return (int)S;
 }

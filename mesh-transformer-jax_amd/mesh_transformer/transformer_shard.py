@@ -85,9 +85,17 @@ class CausalTransformer:
         self.state = {"params": _to_device_tree(tree, self.device), "step": np.array(0)}
         return self
 
+    def invalidate(self):
+        """Forget the packed weights: the next call packs the current parameter tree again.  Needed only after the
+        leaves' memory was written behind torch's back (a raw pointer, another library); assignments to .state and
+        in-place tensor updates are noticed without it."""
+        self._engine = None
+        self._engine_key = None
+
     def engine(self):
         tree = self.state["params"]
-        key = tuple(v.data_ptr() for m in sorted(tree) for _, v in sorted(tree[m].items()))
+        # a leaf is identified by its memory and by torch's version counter, which every in-place update bumps
+        key = tuple((v.data_ptr(), v._version) for m in sorted(tree) for _, v in sorted(tree[m].items()))
         if self._engine is None or key != self._engine_key:
             self._engine = None
             self._engine = Engine(self.config, tree, self.device)
@@ -131,6 +139,8 @@ class CausalTransformer:
         dev = self.device
         with torch.cuda.device(dev):
             ses = eng.session(B, Tcap, Tp, max_pos)
+            if ses.max_pos < max_pos:                   # the kernels would rotate later positions with the last table row
+                raise RuntimeError("rotary tables are shorter than prompt + generated tokens")
             self._ensure_io(ses, G, eng.w.V)
             # --- inputs
             ses.pos0.copy_(torch.from_numpy((-(Tp - (P - 1))).astype(np.int32)))

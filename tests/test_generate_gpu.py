@@ -281,6 +281,30 @@ def test_generate_from_an_8_shard_checkpoint(tmp_path):
     assert np.array_equal(out[0], ref[0])
 
 
+def test_parameter_updates_reach_the_packed_weights():
+    """The packed copies follow the tree: calls on unchanged parameters reuse them, an in-place update of a leaf
+    (no new tensor object, same memory) rebuilds them, and invalidate() forces a rebuild."""
+    from mesh_transformer import sampling
+    params = O.seeded_params(CFG1, 4)
+    ctx = O.left_pad(O.seeded_prompt(4, 1, 40), 64)
+    net = net_for(CFG1, params, sampling.greedy_sample)
+    _, out = net.generate(ctx, [40], 4, {}, return_logits=True)
+    eng = net.engine()
+    _, again = net.generate(ctx, [40], 4, {}, return_logits=True)
+    assert net.engine() is eng and np.array_equal(again[2], out[2])
+    leaf = net.state["params"]["causal_transformer_shard/~/projection_shard/~/linear"]["b"]
+    bump = torch.zeros_like(leaf)
+    bump.view(-1)[123] = 50.0                      # makes token 123 the best one at every step
+    leaf.add_(bump)
+    _, new = net.generate(ctx, [40], 4, {}, return_logits=True)
+    assert net.engine() is not eng
+    assert (new[0][0, :, 0] == 123).all()
+    np.testing.assert_allclose(new[2][0, :1, 0, 123], out[2][0, :1, 0, 123] + 50.0, rtol=0, atol=1e-4)
+    eng2 = net.engine()
+    net.invalidate()
+    assert net.engine() is not eng2
+
+
 def test_sliding_window_evicts_oldest_tokens():
     """ctx not padded (L == P): every decode step drops the oldest real token (layers.py:325-326)."""
     from mesh_transformer import sampling

@@ -236,22 +236,21 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 // out[2i] = x[2i] cos - x[2i+1] sin, out[2i+1] = x[2i+1] cos + x[2i] sin).
 struct inproj_pre {
   int kind;        // 0 q, 1 v, 2 k, 3 fc_in, -1 nothing to store (padding row)
-  float sn, cs;    // rotation of this element (cs = 1, sn = 0 outside the rotary dims)
-  float bias;      // fc_in bias
+  float sn, cs;    // rotation of this element (cs = 1, sn = 0 outside the rotary dims); kind 3: cs is the fc_in bias
   int64_t idx;     // destination element in q / k_cache / v_cache / act
-  int64_t idx_t;   // destination in v_t, or -1
-};
+  int pos_t;       // kind 1 with a transposed copy wanted: the position, i.e. the column of v_t; else -1
+};                 // (kept small: these registers stay live across the whole weight stream of a GEMV)
 
 __device__ __forceinline__ inproj_pre inproj_prepare(const mtj_inproj& ip, const float* __restrict__ b1, int64_t m,
                                                      int64_t n) {
   inproj_pre p;
-  p.sn = 0.f; p.cs = 1.f; p.bias = 0.f; p.idx = 0; p.idx_t = -1;
+  p.sn = 0.f; p.cs = 1.f; p.idx = 0; p.pos_t = -1;
   const int d = ip.n_heads * ip.d_head;
   const int b = (int)(m / ip.Tp), t = (int)(m - (int64_t)b * ip.Tp);
   if (n >= 3 * (int64_t)d) {  // fc_in -> gelu
     const int64_t c = n - 3 * (int64_t)d;
     p.kind = 3;
-    p.bias = b1[c];
+    p.cs = b1[c];
     p.idx = m * ip.ld_act + d + c;
     return p;
   }
@@ -272,8 +271,7 @@ __device__ __forceinline__ inproj_pre inproj_prepare(const mtj_inproj& ip, const
   } else {
     const int slot = pos % ip.Tcap;
     p.idx = (((int64_t)b * ip.n_heads + h) * ip.Tcap + slot) * ip.d_head + e;
-    if (seg == 1 && ip.v_t && pos < ip.ldvt)   // transposed copy, indexed by position like the cache
-      p.idx_t = (((int64_t)b * ip.n_heads + h) * ip.d_head + e) * ip.ldvt + pos;
+    if (seg == 1 && ip.v_t && pos < ip.ldvt) p.pos_t = pos;   // transposed copy, indexed by position like the cache
   }
   return p;
 }
@@ -282,7 +280,7 @@ __device__ __forceinline__ void inproj_finish(const mtj_inproj& ip, const inproj
   const int kv_dtype = ip.kv_dtype;
   if (p.kind < 0) return;
   if (p.kind == 3) {
-    store_as(ip.act, p.idx, gelu_tanh(own + p.bias), ip.act_dtype);
+    store_as(ip.act, p.idx, gelu_tanh(own + p.cs), ip.act_dtype);
     return;
   }
   const float val = own * p.cs + partner * p.sn;
@@ -290,7 +288,10 @@ __device__ __forceinline__ void inproj_finish(const mtj_inproj& ip, const inproj
     store_as(ip.q, p.idx, val, ip.q_dtype);
   } else {
     store_as(p.kind == 1 ? ip.v_cache : ip.k_cache, p.idx, val, kv_dtype);
-    if (p.idx_t >= 0) store_as(ip.v_t, p.idx_t, val, kv_dtype);
+    if (p.pos_t >= 0) {   // idx = ((b*H + h)*Tcap + slot)*dh + e  ->  v_t[((b*H + h)*dh + e)*ldvt + pos]
+      const int64_t bh = p.idx / ((int64_t)ip.Tcap * ip.d_head), e = p.idx % ip.d_head;
+      store_as(ip.v_t, (bh * ip.d_head + e) * ip.ldvt + p.pos_t, val, kv_dtype);
+    }
   }
 }
 

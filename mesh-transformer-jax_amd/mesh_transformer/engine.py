@@ -180,7 +180,10 @@ class Session:
             self.ldvt += 64
         self.x_pf = torch.empty(M, d, dtype=torch.float32, device=dev)
         self.h_pf = torch.empty(M, d, dtype=T, device=dev)
-        self.act_pf = torch.empty(M, d + F, dtype=T, device=dev)
+        # rows of the prefill activations are 128 bytes longer than d + F: with a row pitch that is a multiple of 4 KiB
+        # (40960 bytes at the 6B shape) the 256 rows of an operand tile can compete for the same L2 channels (the
+        # output GEMM alone, M = 16384: 1013 -> 1107 TFLOP/s with the longer rows; inside a layer the gain is ~1 %)
+        self.act_pf = torch.empty(M, d + F + 64, dtype=T, device=dev)[:, :d + F]
         self.q_pf = torch.empty(M * d, dtype=T, device=dev)
         self.vt = torch.zeros(B * H * dh * self.ldvt, dtype=T, device=dev)
         # decode buffers
@@ -242,7 +245,7 @@ class Engine:
         ip.q, ip.q_dtype, ip.kv_dtype = ptr(q), q_dtype, self.w.act_dtype
         ip.k_cache, ip.v_cache = ptr(ses.kc[layer]), ptr(ses.vc[layer])
         ip.v_t, ip.ldvt = (ptr(vt), ses.ldvt) if vt is not None else (None, 0)
-        ip.act, ip.ld_act, ip.act_dtype = ptr(act), act.shape[1], act_dtype
+        ip.act, ip.ld_act, ip.act_dtype = ptr(act), act.stride(0), act_dtype
         return ip
 
     def prefill(self, ses, tokens_rect, Tp, key_limit=None):
@@ -289,8 +292,8 @@ class Engine:
         check(L.mtj_gemm(ptr(h), d, ptr(w.w_in_mm[i]), ptr(w.b1[i]), M, 3 * d + F, d, w.mm_dtype, EPI_INPROJ,
                          None, 0, 0, C.byref(ip), w.alpha_in[i], s))
         check(L.mtj_attn_prefill(ptr(ses.q_pf), ptr(ses.kc[i]), ptr(ses.vt), ptr(pos0), ses.B, self.H, Tp, ses.Tcap,
-                                 self.dh, ses.ldvt, ptr(act), d + F, A, ptr(key_limit), s))
-        check(L.mtj_gemm_splitk(ptr(act), d + F, ptr(w.w_out_mm[i]), ptr(w.b2[i]), M, d, d + F, w.mm_dtype, EPI_RESID,
+                                 self.dh, ses.ldvt, ptr(act), act.stride(0), A, ptr(key_limit), s))
+        check(L.mtj_gemm_splitk(ptr(act), act.stride(0), ptr(w.w_out_mm[i]), ptr(w.b2[i]), M, d, d + F, w.mm_dtype, EPI_RESID,
                                 ptr(x), d, F32, ptr(ses.gemm_work), ses.gemm_work.numel(), w.alpha_out[i], s))
 
     def embed_tok(self, ses):

@@ -123,6 +123,54 @@ def reshard(x, old_shape):
     raise ValueError(f"unimplemented reshard of a {x.ndim}-d leaf")
 
 
+def _fit(x, o, path, shards_in, shards_out):
+    """One leaf: stacked shards x [shards_in, ...] -> the shape of the state's leaf o (resharded if asked)."""
+    shape = tuple(o.shape) if hasattr(o, "shape") else ()
+    if shards_out != shards_in:
+        if shards_out != 1:
+            raise ValueError("this build runs unsharded: shards_out must be 1 (or equal to shards_in)")
+        want = shape if len(shape) == x.ndim else (1,) + shape
+        x = reshard(x, want)
+    if len(shape) != x.ndim and int(np.prod(shape, dtype=np.int64)) == x.size:
+        x = x.reshape(shape)          # the step counter is a scalar here, [shards] in the reference
+    if tuple(x.shape) != shape:
+        raise ValueError(f"Incompatible checkpoints {x.shape} vs {shape} at {'/'.join(path)}")
+    return _from_numpy(x)
+
+
+def read_ckpt_lowmem(pytree, dir, shards_in, shards_out=None, load_opt=True, device=None):
+    """checkpoint.py:178-227: the same result as read_ckpt, read leaf by leaf - piece file by piece file, the same
+    array of every shard, stacked, resharded and put on `device` (the reference spreads the leaves over its devices
+    with jax.device_put; here there is one) - so that the host never holds more than one leaf of every shard at a
+    time (0.8 GB for the 6B embedding instead of the 12 GB tree).  device=None keeps the leaves on the host."""
+    if shards_out is None:
+        shards_out = shards_in
+    skel = {k: v for k, v in pytree.items() if k != "opt_state"}
+    old, paths = tree_flatten(skel)
+    out = []
+    for idx in range(pieces):
+        files = [np.load(os.path.join(dir, f"shard_{s}", f"{idx}.npz"), allow_pickle=False) for s in range(shards_in)]
+        try:
+            names = files[0].files
+            if any(f.files != names for f in files):
+                raise ValueError("shards hold different numbers of arrays")
+            for name in names:
+                if len(out) >= len(old):
+                    raise ValueError(f"checkpoint has more leaves than the state's {len(old)}: only slim checkpoints "
+                                     "(parameters and step, no optimizer state) can be loaded")
+                leaf = _fit(np.stack([f[name] for f in files]), old[len(out)], paths[len(out)], shards_in, shards_out)
+                out.append(leaf.to(device) if device is not None and leaf.ndim > 0 else leaf)
+        finally:
+            for f in files:
+                f.close()
+    if len(out) != len(old):
+        raise ValueError(f"checkpoint has {len(out)} leaves, the state has {len(old)}")
+    state = tree_unflatten(paths, out)
+    if "opt_state" in pytree:
+        state["opt_state"] = pytree["opt_state"]
+    return state
+
+
 def read_ckpt(pytree, dir, shards_in, shards_out=None, load_opt=True):
     """checkpoint.py:135-175.  `pytree` gives the structure and the target shapes (e.g. network.state);
     returns a new state with torch tensors on the host.  Only the inference state is supported: a checkpoint
@@ -140,18 +188,7 @@ def read_ckpt(pytree, dir, shards_in, shards_out=None, load_opt=True):
                          "(parameters and step, no optimizer state) can be loaded")
     out = []
     for o, path, *parts in zip(old, paths, *shards):
-        x = np.stack(parts)
-        shape = tuple(o.shape) if hasattr(o, "shape") else ()
-        if shards_out != shards_in:
-            if shards_out != 1:
-                raise ValueError("this build runs unsharded: shards_out must be 1 (or equal to shards_in)")
-            want = shape if len(shape) == x.ndim else (1,) + shape
-            x = reshard(x, want)
-        if len(shape) != x.ndim and int(np.prod(shape, dtype=np.int64)) == x.size:
-            x = x.reshape(shape)          # the step counter is a scalar here, [shards] in the reference
-        if tuple(x.shape) != shape:
-            raise ValueError(f"Incompatible checkpoints {x.shape} vs {shape} at {'/'.join(path)}")
-        out.append(_from_numpy(x))
+        out.append(_fit(np.stack(parts), o, path, shards_in, shards_out))
     state = tree_unflatten(paths, out)
     if "opt_state" in pytree:
         state["opt_state"] = pytree["opt_state"]

@@ -55,6 +55,12 @@ def test_read_ckpt_folds_8_shards_into_1(tmp_path, dtype):
             got = state["params"][mod][k]
             assert got.dtype == dtype and got.shape == v.shape, (mod, k)
             assert torch.equal(got, v), (mod, k)
+    # leaf by leaf (checkpoint.py:178-227): the same tree
+    low = ckpt.read_ckpt_lowmem(skeleton, d, 8, shards_out=1)
+    assert int(low["step"]) == 383500
+    for mod, leaves in t.items():
+        for k, v in leaves.items():
+            assert low["params"][mod][k].dtype == dtype and torch.equal(low["params"][mod][k], v), (mod, k)
     # same shard count in and out: the stacked tree comes back as it is
     same = ckpt.read_ckpt(stacked, d, 8)
     for mod, leaves in stacked["params"].items():
@@ -71,6 +77,8 @@ def test_read_ckpt_refuses_what_it_cannot_load(tmp_path):
         ckpt.write_ckpt(full, d, s)
     with pytest.raises(ValueError, match="slim"):
         ckpt.read_ckpt({"params": t, "step": np.array(0)}, d, 2, shards_out=1)
+    with pytest.raises(ValueError):          # the optimizer leaves come first in tree order: a shape mismatch or too many
+        ckpt.read_ckpt_lowmem({"params": t, "step": np.array(0)}, d, 2, shards_out=1)
     with pytest.raises(FileNotFoundError):
         ckpt.read_ckpt({"params": t, "step": np.array(0)}, d, 4, shards_out=1)
     bad = dict(CFG, d_model=32)

@@ -581,12 +581,13 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
       if constexpr (ks + 1 < KS) {
         read_frags(st, ks + 1, nxt);
       } else {
-        if (kt + 1 < KT) {
-          __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));       // my part of k-tile kt+1 has landed
-          __builtin_amdgcn_s_waitcnt(wait_lgkmcnt(0));     // my fragment reads of k-tile kt have landed
-          __builtin_amdgcn_s_barrier();
-          read_frags(st ^ 1, 0, nxt);
-        }
+        // Unconditional, also behind the last k-tile (whose "next" fragments are read and dropped): under a
+        // condition, the wait counters of the two paths are merged where they join, and the first MFMAs below
+        // then wait for the fragment reads that were only just issued here.
+        __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));         // my part of k-tile kt+1 has landed
+        __builtin_amdgcn_s_waitcnt(wait_lgkmcnt(0));       // my fragment reads of k-tile kt have landed
+        __builtin_amdgcn_s_barrier();
+        read_frags(st ^ 1, 0, nxt);
       }
       __builtin_amdgcn_sched_barrier(0);
       for_stages<0, WM * WN>([&](auto Q_) {

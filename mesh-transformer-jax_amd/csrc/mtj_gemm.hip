@@ -22,6 +22,9 @@ template <> struct mma<bf16_t> {
   __device__ static __forceinline__ void run(floatx16& c, const frag& a, const frag& b) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
   }
+  __device__ static __forceinline__ void run16(floatx4& c, const frag& a, const frag& b) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, c, 0, 0, 0);
+  }
 };
 template <> struct mma<f16_t> {
   static constexpr int EPC = 8;
@@ -33,6 +36,9 @@ template <> struct mma<f16_t> {
   }
   __device__ static __forceinline__ void run(floatx16& c, const frag& a, const frag& b) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.v, b.v, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ void run16(floatx4& c, const frag& a, const frag& b) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.v, b.v, c, 0, 0, 0);
   }
 };
 template <> struct mma<float> {
@@ -112,12 +118,15 @@ __device__ __forceinline__ void for_stages(F&& f) {
 // fc_in columns: 16 bias values; rotary q/k columns: 8 sines then 8 cosines
 struct epi_ops { floatx4 o[4]; };
 
-// Epilogue of a workgroup tile whose wavefront (wm, wn) holds WM x WN accumulator tiles of 32x32; accumulator
-// register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32].  `smem` (the operand staging area, no longer
-// needed) must hold 2*BM ints and one 32x36 float patch per wavefront.
-template <int EPI, int WAVES_M, int WAVES_N, int WM, int WN>
-__device__ __forceinline__ void epilogue(const gemm_args& a, void* out, floatx16 (&acc)[WM][WN], unsigned char* smem, int m0,
-                                         int n0) {
+// Epilogue of a workgroup tile whose wavefront (wm, wn) holds WM x WN accumulator tiles of 32x32.  `smem` (the
+// operand staging area, no longer needed) must hold 2*BM ints and one 32x36 float patch per wavefront.
+// Two accumulator layouts:
+//   MI16 false  acc is floatx16[WM][WN] from 32x32 MFMAs: register v of lane l holds C[8*(v/4) + 4*(l/32) + v%4][l%32];
+//   MI16 true   acc is floatx4[2*WM][2*WN] from 16x16x32 MFMAs issued with the WEIGHT fragment as the first operand:
+//               register v of lane l of block (i, j) holds C[16*i + l%16][16*j + 4*(l/16) + v], four consecutive
+//               columns of one row, so stores are 8 or 16 bytes per lane.
+template <int EPI, int WAVES_M, int WAVES_N, int WM, int WN, bool MI16 = false, class ACC>
+__device__ __forceinline__ void epilogue(const gemm_args& a, void* out, ACC& acc, unsigned char* smem, int m0, int n0) {
   constexpr int NT = WAVES_M * WAVES_N * 64, BM = WAVES_M * WM * 32;
   constexpr int PS = 36;   // patch row stride in floats: 16-byte aligned rows, and 16-byte reads of 8 lanes hit distinct banks
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -130,6 +139,58 @@ __device__ __forceinline__ void epilogue(const gemm_args& a, void* out, floatx16
     constexpr int BN = WAVES_N * WN * 32;
     __syncthreads();                                       // every wavefront is done with the operand tiles
     float* red = reinterpret_cast<float*>(smem);           // [WAVES_N][BM][2]
+    if constexpr (MI16) {
+      // a lane holds 4 columns of each of the 2*WN column blocks of its row; a row is completed by the four lanes
+      // l%16 + 16*q, then by the WAVES_N wavefronts through LDS
+      const int r16 = lane & 15, q16 = lane >> 4;
+      float bias[2 * WN][4];
+      bool ok[2 * WN][4];
+#pragma unroll
+      for (int j = 0; j < 2 * WN; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int n = n0 + (wn * WN * 2 + j) * 16 + 4 * q16 + v;
+          ok[j][v] = n < a.N;
+          bias[j][v] = (a.bias && ok[j][v]) ? a.bias[n] : 0.f;
+        }
+      for_tiles<0, 0, 2 * WM, 1>([&](auto I_, auto) {
+        constexpr int i = decltype(I_)::value;
+        const int r = (wm * WM * 2 + i) * 16 + r16;
+        const int m = m0 + r;
+        float val[2 * WN][4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 2 * WN; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            val[j][v] = ok[j][v] ? acc[i][j][v] * a.alpha + bias[j][v] : -INFINITY;
+            mx = fmaxf(mx, val[j][v]);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        float sm = 0.f;
+        if (mx != -INFINITY) {
+#pragma unroll
+          for (int j = 0; j < 2 * WN; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) sm += __expf(val[j][v] - mx);      // exp(-inf) = 0 for columns beyond N
+        }
+        sm += __shfl_xor(sm, 16);
+        sm += __shfl_xor(sm, 32);
+        if (m < a.M) {
+          const int t = a.target[m];
+#pragma unroll
+          for (int j = 0; j < 2 * WN; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+              if (n0 + (wn * WN * 2 + j) * 16 + 4 * q16 + v == t) a.tlogit[m] = val[j][v];
+        }
+        if (q16 == 0) {
+          red[(wn * BM + r) * 2] = mx;
+          red[(wn * BM + r) * 2 + 1] = sm;
+        }
+      });
+    } else
     for_tiles<0, 0, WM, 1>([&](auto I_, auto) {
       constexpr int i = decltype(I_)::value;
       float val[WN][16];
@@ -251,8 +312,17 @@ __device__ __forceinline__ void epilogue(const gemm_args& a, void* out, floatx16
       epi_ops nxt = cur;
       if constexpr (nj < WN) nxt = load_ops(ni, nj);
       const col_info c = column(j);
+      if constexpr (MI16) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) patch[(8 * (v / 4) + 4 * fg + (v % 4)) * PS + fr] = acc[i][j][v] * a.alpha;
+        for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj)
+            *reinterpret_cast<floatx4*>(patch + (ii * 16 + (lane & 15)) * PS + jj * 16 + 4 * (lane >> 4)) =
+                acc[2 * i + ii][2 * j + jj] * a.alpha;
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) patch[(8 * (v / 4) + 4 * fg + (v % 4)) * PS + fr] = acc[i][j][v] * a.alpha;
+      }
       __builtin_amdgcn_wave_barrier();
       float val[16];
 #pragma unroll
@@ -296,6 +366,47 @@ __device__ __forceinline__ void epilogue(const gemm_args& a, void* out, floatx16
         }
       }
       cur = nxt;
+    });
+  } else if constexpr (MI16) {
+    // four consecutive columns per lane: 16-byte (float32) or 8-byte (16-bit) accesses when the rows of `out` allow it
+    const int r16 = lane & 15, q16 = lane >> 4;
+    const int esz = (EPI == MTJ_EPI_RESID || a.out_dtype == MTJ_F32) ? 4 : 2;
+    const bool vec = a.ldo % 4 == 0 && (reinterpret_cast<uintptr_t>(out) % (4 * esz)) == 0;
+    for_tiles<0, 0, 1, 2 * WN>([&](auto, auto J_) {
+      constexpr int j = decltype(J_)::value;
+      const int nb = n0 + (wn * WN * 2 + j) * 16 + 4 * q16;
+      float bias[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) bias[v] = (a.bias && nb + v < a.N) ? a.bias[nb + v] : 0.f;
+      const bool full = vec && nb + 3 < a.N;
+      for_tiles<0, 0, 2 * WM, 1>([&](auto I_, auto) {
+        constexpr int i = decltype(I_)::value;
+        const int m = m0 + (wm * WM * 2 + i) * 16 + r16;
+        if (m >= a.M) return;
+        const int64_t idx = (int64_t)m * a.ldo + nb;
+        float val[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) val[v] = acc[i][j][v] * a.alpha + bias[v];
+        if (full) {
+          if (EPI == MTJ_EPI_RESID) {
+            floatx4* o = reinterpret_cast<floatx4*>(reinterpret_cast<float*>(out) + idx);
+            const floatx4 old = *o;
+            *o = floatx4{old.x + val[0], old.y + val[1], old.z + val[2], old.w + val[3]};
+          } else if (a.out_dtype == MTJ_F32) {
+            *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(out) + idx) = floatx4{val[0], val[1], val[2], val[3]};
+          } else {
+            *reinterpret_cast<uint32x2*>(reinterpret_cast<uint16_t*>(out) + idx) =
+                uint32x2{pack_16x2(val[0], val[1], a.out_dtype), pack_16x2(val[2], val[3], a.out_dtype)};
+          }
+        } else {
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (nb + v < a.N) {
+              if (EPI == MTJ_EPI_RESID) reinterpret_cast<float*>(out)[idx + v] += val[v];
+              else store_as(out, idx + v, val[v], a.out_dtype);
+            }
+        }
+      });
     });
   } else {
     for_tiles<0, 0, WM, WN>([&](auto I_, auto J_) {
@@ -472,31 +583,36 @@ typedef __attribute__((address_space(3))) void* lds_ptr;
 constexpr int wait_vmcnt(int n) { return (n & 0xf) | (((n >> 4) & 3) << 14) | (0x7 << 4) | (0xf << 8); }
 constexpr int wait_lgkmcnt(int n) { return 0xf | (3 << 14) | (0x7 << 4) | ((n & 0xf) << 8); }
 
-// bf16, 256x256 workgroup tile, 8 wavefronts of 128x64, K step 64, two LDS stages of 64 KiB.
+// 16-bit operands, 256x256 workgroup tile, 8 wavefronts of 128x64, K step 64, two LDS stages of 64 KiB,
+// v_mfma_f32_16x16x32 (under the board's power limit it sustains a higher clock than the 32x32x16 form: 1820 against
+// 1570 TFLOP/s in a register-only loop on random float16 data).
 //
 // The memory pipeline writes the operand tiles straight into LDS (buffer_load_dwordx4 ... lds: 64 lanes x
-// 16 bytes land at consecutive LDS addresses), so there are no staging registers, no ds_write and the loads
-// of k-tile kt+2 are in flight while k-tile kt+1 waits in LDS.  A tile row is 128 bytes = 8 chunks; LDS
-// position (row, c) holds chunk c ^ ((row >> 1) & 7) of the row, which each lane arranges by choosing its
-// global address, and which makes the 16-byte fragment reads of 16 consecutive rows hit 16 distinct bank
-// groups without padding.  One barrier per k-tile, placed before the last of the four MFMA steps: behind it
-// k-tile kt+1 is visible to everyone and k-tile kt has been read by everyone, so the first fragments of kt+1
-// are fetched under the last MFMAs of kt and the stage of kt is handed to the loads of kt+2.  Those eight
-// loads per wavefront are issued one per two MFMAs (a burst would stall the wavefront on the address queue
-// with its MFMAs behind it).  Rows beyond M or N are outside the buffer resource and read as zero.
+// 16 bytes land at consecutive LDS addresses), so there are no staging registers and no ds_write.  A tile row is
+// 128 bytes = 8 chunks; LDS position (row, c) holds chunk c ^ ((row >> 1) & 7) of the row, which each lane arranges
+// by choosing its global address, and which makes the 16-byte fragment reads of 16 consecutive rows hit 16 distinct
+// bank groups without padding.  Rows beyond M or N are outside the buffer resource and read as zero.
+//
+// The two wavefronts of a SIMD (wave w and w + 4) never compete for the matrix pipe: a k-tile is eight clusters,
+// memory clusters (fragment reads from LDS, two global->LDS loads, the wait for an older load) alternating with
+// MFMA clusters (one quarter of the wavefront's tile: 64 rows x 32 columns x 64 k = 16 MFMAs), every cluster ends
+// in a workgroup barrier, and wavefronts 4..7 run one cluster behind wavefronts 0..3, so that at any time four
+// wavefronts multiply while the other four read.  Operands are loaded in four sets per k-tile (A rows / W rows
+// of the first and second half of every wavefront's tile) in the order the clusters consume them, each set into
+// the place of the same set two k-tiles earlier as soon as both groups have read that one; every load is issued
+// nine to ten clusters before its first reader.  Loads for k-tiles beyond the range re-read the last k-tile
+// (the stage they land in is not read again), which keeps the wait counts the same in every k-tile.
 template <typename T, int EPI>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
   static_assert(sizeof(T) == 2, "16-bit operands");
-  constexpr int WAVES_M = 2, WAVES_N = 4, WM = 4, WN = 2, NT = 512, BM = 256, BN = 256, BK = 64, NST = 2;
-  constexpr int ROWB = BK * 2, CPR = BK / 8, OPB = BM * ROWB, STAGEB = 2 * OPB;
-  constexpr int LOADS = BM * CPR / NT, ROWS_PER_LOAD = NT / CPR, KS = BK / 16;
-  static_assert(WM * WN == 2 * LOADS, "one load per two MFMAs");
+  constexpr int WAVES_M = 2, WAVES_N = 4, WM = 4, WN = 2, BM = 256, BN = 256, BK = 64;
+  constexpr int ROWB = BK * 2, OPB = BM * ROWB, STAGEB = 2 * OPB;
   extern __shared__ __align__(16) unsigned char smem[];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
-  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-  const int fr = lane & 31, fg = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const int fr = lane & 15, fq = lane >> 4;
 
   // tile id: as in gemm_kernel (contiguous tile ranges per XCD, groups of 8 row-tiles)
   const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
@@ -521,94 +637,139 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
       const_cast<T*>(tile_a), 0, (int)((((int64_t)rows_a - 1) * a.lda + a.K) * 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T*>(tile_b), 0, (int)((((int64_t)rows_b - 1) * a.K + a.K) * 2), 0x00020000);
-  auto swz = [](int row) { return (row >> 1) & 7; };
-  const int lr = tid / CPR;                                  // my row inside one load's 64 rows
-  const int lc = ((tid % CPR) ^ swz(lr)) * 16;               // byte offset of the chunk I fetch for my LDS position
-  const int voff_a = (int)((int64_t)lr * a.lda * 2) + lc, voff_b = (int)((int64_t)lr * a.K * 2) + lc;
-  const int pass_a = (int)((int64_t)ROWS_PER_LOAD * a.lda * 2), pass_b = (int)((int64_t)ROWS_PER_LOAD * a.K * 2);
+
+  // a wavefront load = 8 rows x 128 bytes at 1 KiB of consecutive LDS; lane l fetches, for LDS position l % 8 of
+  // row l / 8, chunk (l % 8) ^ swizzle(row): every row base used below is a multiple of 8 whose bit 3 is wave & 1
+  const int chunk = (lane & 7) ^ ((lane >> 4) & 3) ^ ((wave & 1) << 2);
+  const int voff_a = (int)((int64_t)(lane >> 3) * a.lda * 2) + chunk * 16;
+  const int voff_b = (int)((int64_t)(lane >> 3) * a.K * 2) + chunk * 16;
+  // my two loads of a set: A rows wave*8 and 128 + wave*8 (+64 for the second-half set), W rows
+  // (wave/4)*64 + (wave%4)*8 and 128 more (+32 for the second-half set)
+  const int ra0 = wave * 8, rb0 = (wave >> 2) * 64 + (wave & 3) * 8;
 
   // my K range (split-K: blockIdx.y; the whole of K otherwise), in k-tiles
   const int kt0 = (int)((int64_t)blockIdx.y * (a.K / BK) / a.splits);
   const int KT = (int)((int64_t)(blockIdx.y + 1) * (a.K / BK) / a.splits) - kt0;
 
-  // load number l of k-tile kt of my range: l < LOADS fetches rows [l*64, l*64+64) of A, the others of W
-  auto issue_one = [&](int st, int kt, auto L_) {
-    constexpr int l = decltype(L_)::value, part = l / LOADS, i = l % LOADS;
-    unsigned char* dst = smem + st * STAGEB + part * OPB + i * (NT * 16) + wave_s * 1024;
-    if (part == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr)dst, 16, voff_a, (kt0 + kt) * ROWB + i * pass_a, 0, 0);
-    else __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr)dst, 16, voff_b, (kt0 + kt) * ROWB + i * pass_b, 0, 0);
+  // set 0: A first half, 1: W first half, 2: W second half, 3: A second half
+  auto issue = [&](int st, int kt, auto SET_) {
+    constexpr int set = decltype(SET_)::value;
+    const int koff = (kt0 + (kt < KT ? kt : KT - 1)) * ROWB;
+    if constexpr (set == 0 || set == 3) {
+      const int r = ra0 + (set == 3 ? 64 : 0);
+      unsigned char* d = smem + st * STAGEB + r * ROWB;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr)d, 16, voff_a, koff + (int)((int64_t)r * a.lda * 2), 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr)(d + 128 * ROWB), 16, voff_a,
+                                               koff + (int)((int64_t)(r + 128) * a.lda * 2), 0, 0);
+    } else {
+      const int r = rb0 + (set == 2 ? 32 : 0);
+      unsigned char* d = smem + st * STAGEB + OPB + r * ROWB;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr)d, 16, voff_b, koff + (int)((int64_t)r * a.K * 2), 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr)(d + 128 * ROWB), 16, voff_b,
+                                               koff + (int)((int64_t)(r + 128) * a.K * 2), 0, 0);
+    }
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+
+  floatx4 acc[2 * WM][2 * WN];
+#pragma unroll
+  for (int i = 0; i < 2 * WM; ++i)
+#pragma unroll
+    for (int j = 0; j < 2 * WN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  issue(0, 0, I0{}); issue(0, 0, I1{}); issue(0, 0, I2{}); issue(0, 0, I3{});
+  issue(1, 1, I0{}); issue(1, 1, I1{});
+
+  // fragments of a 16x16x32 MFMA: lane (fr, fq) supplies elements [8*fq, 8*fq + 8) of the 32-wide k-step of row fr
+  int xo[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) xo[ks] = ((4 * ks + fq) ^ ((fr >> 1) & 7)) * 16;
+  const int a_row = (wm * 128 + fr) * ROWB, b_row = OPB + (wn * 64 + fr) * ROWB;
+  typename mma<T>::frag fa[2 * WM][2], fb[2 * WN][2];
+  // read number n = 4*ks + i of A half h (row blocks 4h .. 4h+3), reads [n_lo, n_hi)
+  auto read_a = [&](int st, int h, int n_lo, int n_hi) {
+#pragma unroll
+    for (int n = 0; n < 8; ++n)
+      if (n >= n_lo && n < n_hi)
+        fa[4 * h + (n & 3)][n >> 2] =
+            mma<T>::load(reinterpret_cast<const T*>(smem + st * STAGEB + a_row + (4 * h + (n & 3)) * 16 * ROWB + xo[n >> 2]));
+  };
+  auto read_b = [&](int st, int h) {
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+      fb[2 * h + (n & 1)][n >> 1] =
+          mma<T>::load(reinterpret_cast<const T*>(smem + st * STAGEB + b_row + (2 * h + (n & 1)) * 16 * ROWB + xo[n >> 1]));
+  };
+  // 64 rows (A half ha) x 32 columns (W half hb) x 64: the two MFMAs of an accumulator are 8 instructions apart
+  auto multiply = [&](auto HA_, auto HB_) {
+    constexpr int ha = decltype(HA_)::value, hb = decltype(HB_)::value;
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) mma<T>::run16(acc[4 * ha + i][2 * hb + j], fb[2 * hb + j][ks], fa[4 * ha + i][ks]);
+    __builtin_amdgcn_s_setprio(0);
+  };
+  // end of a memory cluster: the set that the next memory cluster reads was issued four sets ago
+  auto landed = [&]() { __builtin_amdgcn_s_waitcnt(wait_vmcnt(8)); };
+  auto cluster_end = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
   };
 
-  floatx16 acc[WM][WN];
-#pragma unroll
-  for (int i = 0; i < WM; ++i)
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-  for_stages<0, 2 * LOADS>([&](auto L_) { issue_one(0, 0, L_); });
-  if (KT > 1) for_stages<0, 2 * LOADS>([&](auto L_) { issue_one(1, 1, L_); });
-
-  // fragment addresses: lane (fr, fg) reads chunk (2*ks + fg) ^ swz(fr) of its row in k-step ks
-  int xo[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) xo[ks] = ((2 * ks + fg) ^ swz(fr)) * 16;
-  const int a_row = (wm * WM * 32 + fr) * ROWB, b_row = OPB + (wn * WN * 32 + fr) * ROWB;
-  typename mma<T>::frag fa[2][WM], fb[2][WN];
-  auto read_frags = [&](int st, int ks, int slot) {
-    const unsigned char* p = smem + st * STAGEB + xo[ks];
-#pragma unroll
-    for (int i = 0; i < WM; ++i) fa[slot][i] = mma<T>::load(reinterpret_cast<const T*>(p + a_row + i * 32 * ROWB));
-#pragma unroll
-    for (int j = 0; j < WN; ++j) fb[slot][j] = mma<T>::load(reinterpret_cast<const T*>(p + b_row + j * 32 * ROWB));
-  };
-  if (KT > 1) __builtin_amdgcn_s_waitcnt(wait_vmcnt(2 * LOADS));
-  else __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
+  landed();
   __builtin_amdgcn_s_barrier();
-  read_frags(0, 0, 0);
+  if (wm) __builtin_amdgcn_s_barrier();        // wavefronts 4..7 start one cluster late
+  __builtin_amdgcn_sched_barrier(0);
+  read_a(0, 0, 0, 6);
 
+  // k-tile kt in stage st; fragment reads per memory cluster: 6 + 6 + 4 + 8
   auto k_tile = [&](int kt, auto ST_) {
     constexpr int st = decltype(ST_)::value;
-    for_stages<0, KS>([&](auto KS_) {
-      constexpr int ks = decltype(KS_)::value, cur = ks & 1, nxt = cur ^ 1;
-      // loads of k-tile kt+2 go out behind the barrier of k-tile kt: the first half under the last step of kt,
-      // the second half under the first step of kt+1 (where they are the loads "of" kt-1+2)
-      constexpr bool first_half = ks == KS - 1, second_half = ks == 0;
-      constexpr int l_st = first_half ? st : st ^ 1;
-      const int l_kt = first_half ? kt + NST : kt - 1 + NST;
-      const bool go = first_half ? (kt + NST < KT) : (kt >= 1 && kt - 1 + NST < KT);
-      if constexpr (ks + 1 < KS) {
-        read_frags(st, ks + 1, nxt);
-      } else {
-        // Unconditional, also behind the last k-tile (whose "next" fragments are read and dropped): under a
-        // condition, the wait counters of the two paths are merged where they join, and the first MFMAs below
-        // then wait for the fragment reads that were only just issued here.
-        __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));         // my part of k-tile kt+1 has landed
-        __builtin_amdgcn_s_waitcnt(wait_lgkmcnt(0));       // my fragment reads of k-tile kt have landed
-        __builtin_amdgcn_s_barrier();
-        read_frags(st ^ 1, 0, nxt);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      for_stages<0, WM * WN>([&](auto Q_) {
-        constexpr int q = decltype(Q_)::value, i = q / WN, j = q % WN;
-        mma<T>::run(acc[i][j], fa[cur][i], fb[cur][j]);
-        if constexpr ((first_half || second_half) && (q & 1)) {
-          __builtin_amdgcn_sched_barrier(0);
-          if (go) issue_one(l_st, l_kt, std::integral_constant<int, (first_half ? 0 : LOADS) + q / 2>{});
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      });
-      __builtin_amdgcn_sched_barrier(0);
-    });
+    read_a(st, 0, 6, 8);
+    read_b(st, 0);
+    issue(st ^ 1, kt + 1, I2{});
+    landed();
+    cluster_end();
+    multiply(I0{}, I0{});
+    cluster_end();
+    read_b(st, 1);
+    issue(st ^ 1, kt + 1, I3{});
+    landed();
+    cluster_end();
+    multiply(I0{}, I1{});
+    cluster_end();
+    read_a(st, 1, 0, 8);
+    issue(st, kt + 2, I0{});
+    landed();
+    cluster_end();
+    multiply(I1{}, I0{});
+    cluster_end();
+    read_a(st ^ 1, 0, 0, 6);                   // of k-tile kt+1
+    issue(st, kt + 2, I1{});
+    landed();
+    cluster_end();
+    multiply(I1{}, I1{});
+    cluster_end();
   };
-  for (int kt = 0; kt < KT; kt += NST)
-    for_stages<0, NST>([&](auto S_) {
-      if (kt + decltype(S_)::value < KT) k_tile(kt + decltype(S_)::value, S_);
-    });
+  int kt = 0;
+  for (; kt + 1 < KT; kt += 2) {
+    k_tile(kt, I0{});
+    k_tile(kt + 1, I1{});
+  }
+  if (kt < KT) k_tile(kt, I0{});
+  __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));   // the surplus loads land before this workgroup's LDS is given away
+  if (!wm) __builtin_amdgcn_s_barrier();
+  __syncthreads();                             // every wavefront's loads have landed: the epilogue may reuse the stages
 
   void* out = a.splits > 1 ? (void*)(reinterpret_cast<float*>(a.out) + blockIdx.y * a.split_stride) : a.out;
-  epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, out, acc, smem, m0, n0);
+  epilogue<EPI, WAVES_M, WAVES_N, WM, WN, true>(a, out, acc, smem, m0, n0);
 }
 
 template <typename T, int EPI>

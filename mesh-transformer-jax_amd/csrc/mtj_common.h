@@ -221,11 +221,16 @@ __device__ __forceinline__ floatx4 mtj_merge_partials(const float* __restrict__ 
 }
 
 // jax.nn.gelu(approximate=True): 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3).
-// 0.5 (1 + tanh(u)) = 1 / (1 + exp(-2u)); evaluated with the hardware exp2 and reciprocal (a few ulp).
+// 0.5 (1 + tanh(u)) = 1 / (1 + exp(-2u)) = 1 / (1 + 2^(x (k1 + k2 x^2))) with k1 = -2 log2(e) sqrt(2/pi) and
+// k2 = 0.044715 k1: three multiplications, one fma, one addition, v_exp_f32 and v_rcp_f32 (about 1 ulp each).  The
+// plain spelling x / (1 + expf(-2u)) compiles to a correctly rounded division of about twenty instructions, which made
+// the fc_in columns of the prefill epilogue twice as expensive.  For very negative x the power overflows to +inf and the
+// result is -0; for large x it underflows to 0 and the result is x.
 __device__ __forceinline__ float gelu_tanh(float x) {
-  const float c = 0.7978845608028654f;
-  const float u = c * (x + 0.044715f * x * x * x);
-  return __fdividef(x, 1.0f + __expf(-2.0f * u));
+  const float k1 = -2.3022082f;        // -2 * 1.4426950408889634 * 0.7978845608028654
+  const float k2 = -0.10294324f;       // k1 * 0.044715
+  const float p = fmaf(x * x, k2, k1);
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * p));
 }
 
 // ---------------------------------------------------------------- fused input-projection epilogue

@@ -1,5 +1,6 @@
 // Attention: MFMA flash-style prefill over a left-padded rectangle, and one-token decode over the K/V window.
 #include "mtj_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -358,6 +359,312 @@ __global__ __launch_bounds__(NW * 64) void attn_prefill_kernel(const T* __restri
 }
 
 // ------------------------------------------------------------------------------------------------
+// Prefill for 16-bit types at d_head 256: the same mathematics and the same lane layout as attn_prefill_kernel (one
+// lane owns one query, S^T = K Q^T, O^T = V^T P^T, K rows permuted so that the scores land in the operand layout of the
+// second product), but each block of 32 queries is worked on by a PAIR of wavefronts that share a SIMD (wave w and
+// w + 4 of an 8-wavefront workgroup, 128 queries per workgroup):
+//   the score wavefront (w < 4) holds Q and computes the scores of key tile i, their running maximum and the rescale
+//     factor, and hands score - maximum to its partner through LDS;
+//   the value wavefront (w + 4) holds the output accumulator and the running sum, turns the scores of tile i-1 into
+//     probabilities (the exponentials) and multiplies them with V^T; it also issues every global -> LDS load.
+// An iteration is two phases separated by workgroup barriers: [scores of tile i | exponentials of tile i-1], then
+// [maximum of tile i | P V of tile i-1], so the two wavefronts of a SIMD take turns on the matrix pipe and each one's
+// vector arithmetic runs under the other's MFMAs; with one wavefront per SIMD doing all of it in sequence the matrix
+// pipe was busy a quarter of the time.  K and V^T tiles of 32 keys go global -> LDS without passing through registers
+// (buffer_load ... lds), four stages each, requested three (K) and two (V^T) tiles ahead; rows are unpadded and the
+// 16-byte chunks of a row are xor-swizzled (K: low four bits of the chunk index with the row, V^T: the two bits with
+// (row / 4) % 4) so that the fragment reads of 16 consecutive rows hit 16 distinct bank groups.  Loads beyond the last
+// tile re-read the last tile (into a stage nobody reads again), which keeps the wait count the same in every iteration.
+constexpr int PP_STAGES = 4, PP_KTILE = 32 * 256 * 2, PP_VTILE = 256 * 32 * 2;
+constexpr int PP_LDS_K = 0, PP_LDS_V = PP_STAGES * PP_KTILE, PP_LDS_S = PP_LDS_V + PP_STAGES * PP_VTILE;
+constexpr int PP_LDS_A = PP_LDS_S + 4 * 4096, PP_LDS_F = PP_LDS_A + 4 * 512, PP_LDS_BYTES = PP_LDS_F + 64;
+
+// sum of eight 16-bit probabilities as the second product will see them (after rounding), added to acc
+template <typename T> struct psum;
+template <> struct psum<f16_t> {
+  __device__ static __forceinline__ float run(const typename mma<f16_t>::frag& f, float acc) {
+    const f16x2 one = {(f16_t)1.f, (f16_t)1.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_fdot2(f16x2{f.v[2 * j], f.v[2 * j + 1]}, one, acc, false);
+    return acc;
+  }
+};
+template <> struct psum<bf16_t> {
+  __device__ static __forceinline__ float run(const typename mma<bf16_t>::frag& f, float acc) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc += (float)f.v[j];
+    return acc;
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(512) void attn_prefill_pair_kernel(const T* __restrict__ q, const T* __restrict__ kc,
+                                                                const T* __restrict__ vt, const int32_t* __restrict__ pos0,
+                                                                int H, int Tp, int Tcap, int64_t ldvt, T* __restrict__ out,
+                                                                int64_t ld_out, int nseq, int nqblk,
+                                                                const int32_t* __restrict__ key_limit) {
+  static_assert(sizeof(T) == 2, "16-bit types");
+  constexpr int DH = 256, BKV = 32, BQ = 128, KS = DH / 16, NBLK = DH / 32;
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int pw = wave & 3;                      // which 32 queries of the workgroup
+  const bool value_role = wave >= 4;
+  const int fr = lane & 31, fg = lane >> 5;
+  const int hb = blockIdx.x % (H * nseq), qblk = blockIdx.x / (H * nseq);
+  const int h = hb % H, b = hb / H;
+  const int qt0 = (nqblk - 1 - qblk) * BQ;      // longest workgroups first
+  const int t = qt0 + pw * 32 + fr;             // this lane's query (rectangle index)
+  const int64_t bh = (int64_t)b * H + h;
+
+  float* sx = reinterpret_cast<float*>(smem + PP_LDS_S + pw * 4096) + lane * 4;   // + v4 * 256 floats
+  float* ax = reinterpret_cast<float*>(smem + PP_LDS_A + pw * 512) + lane;        // rescale factor, + 64: minus the maximum
+  int* fx = reinterpret_cast<int*>(smem + PP_LDS_F) + pw;
+  const float sc2 = rsqrtf((float)DH) * 1.4426950408889634f;   // 1/sqrt(dh) * log2(e): probabilities are 2^(s*sc2 - max)
+
+  // Requests that do not depend on the sequence's padding go out before it is known: Q, and the first three K tiles and
+  // two V^T tiles (a row or column index beyond the buffers is clamped into them; such a tile is never read).
+  typename mma<T>::frag qf[KS];
+  const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(kc + bh * Tcap * DH), 0, (int)((int64_t)Tcap * DH * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(vt + bh * DH * ldvt), 0, (int)((int64_t)DH * ldvt * 2), 0x00020000);
+  // global -> LDS loads.  K tile: 32 rows x 512 bytes = 16 wavefront loads of 2 rows, load j = 4*wb + jj; lane l fills
+  // position l % 32 of row 2j + l / 32 with chunk (p & 16) | ((p & 15) ^ (row & 15)).  V^T tile: 256 rows x 64 bytes =
+  // 16 loads of 16 rows; lane l fills position l % 4 of row 16j + l / 4 with chunk (l % 4) ^ ((row / 4) % 4).
+  const int wb = wave & 3;
+  int k_row[4], k_chunk[4], v_off[4];
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) {
+    const int j = 4 * wb + jj;
+    k_row[jj] = 2 * j + (lane >> 5);
+    const int kp_l = lane & 31;
+    k_chunk[jj] = ((kp_l & 16) | ((kp_l & 15) ^ (k_row[jj] & 15))) * 16;
+    const int vrow_l = 16 * j + (lane >> 2);
+    v_off[jj] = (int)((int64_t)vrow_l * ldvt * 2) + (((lane & 3) ^ ((vrow_l >> 2) & 3)) * 16);
+  }
+  auto issue_k1 = [&](int stage_tile, int tile, auto JJ_) {
+    constexpr int jj = decltype(JJ_)::value;
+    unsigned char* dst = smem + PP_LDS_K + (stage_tile & (PP_STAGES - 1)) * PP_KTILE + wb * 4096 + jj * 1024;
+    const int row = tile * BKV + k_row[jj];                 // rows beyond the last key are masked by their readers
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)dst, 16, (row < Tcap ? row : Tcap - 1) * 512 + k_chunk[jj], 0, 0, 0);
+  };
+  auto issue_v1 = [&](int stage_tile, int tile, auto JJ_) {
+    constexpr int jj = decltype(JJ_)::value;
+    unsigned char* dst = smem + PP_LDS_V + (stage_tile & (PP_STAGES - 1)) * PP_VTILE + wb * 4096 + jj * 1024;
+    const int64_t col = (int64_t)tile * BKV + BKV <= ldvt ? (int64_t)tile * BKV : ldvt - BKV;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)dst, 16, v_off[jj] + (int)col * 2, 0, 0, 0);
+  };
+  using J0 = std::integral_constant<int, 0>;
+  using J1 = std::integral_constant<int, 1>;
+  using J2 = std::integral_constant<int, 2>;
+  using J3 = std::integral_constant<int, 3>;
+  auto issue_k = [&](int st, int tile) { issue_k1(st, tile, J0{}); issue_k1(st, tile, J1{}); issue_k1(st, tile, J2{}); issue_k1(st, tile, J3{}); };
+  auto issue_v = [&](int st, int tile) { issue_v1(st, tile, J0{}); issue_v1(st, tile, J1{}); issue_v1(st, tile, J2{}); issue_v1(st, tile, J3{}); };
+  if (value_role) {
+    issue_k(0, 0); issue_v(0, 0); issue_k(1, 1); issue_v(1, 1); issue_k(2, 2);
+  } else {
+    const int tq = (t < Tp) ? t : Tp - 1;
+    const T* qp = q + (bh * Tp + tq) * DH + fg * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = mma<T>::load(qp + ks * 16);
+  }
+
+  const int p0 = pos0[b];                       // <= 0: minus the number of padding rows
+  const int qpos = (t < Tp) ? t + p0 : -1;      // its position; < 0 = padding / out of range
+  const int klim = key_limit ? key_limit[b] : 0x7fffffff;
+  const int qsee = qpos < klim ? qpos : klim;   // last key this query may see
+  const int last_t = (qt0 + BQ - 1 < Tp - 1) ? qt0 + BQ - 1 : Tp - 1;
+  const int kmax = last_t + p0;                 // last key any query of this workgroup may see
+  const int klast = Tp - 1 + p0;                // last key position that exists for this sequence
+  const int wave_last = qt0 + pw * 32 + 31 + p0;     // last key this pair may see
+  const int wave_first0 = (qt0 + pw * 32 + 31 < Tp) ? qt0 + pw * 32 + p0 : -1;
+  const int wave_first = wave_first0 < klim ? wave_first0 : klim;
+  const int ntiles = (kmax >= 0) ? kmax / BKV + 1 : 0;
+
+  if (!value_role) {
+    // ---------------- score wavefront
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) mma<T>::pin(qf[ks]);   // pinned, or Q is re-loaded inside the key loop
+    // row fr of an S^T block is key krow: rows {0-3, 4-7, 8-11, 12-15} <- keys {0-3, 8-11, 4-7, 12-15} (+16)
+    const int krow = 16 * (fr >> 4) + 8 * ((fr >> 2) & 1) + 4 * ((fr >> 3) & 1) + (fr & 3);
+    const int kx = (krow & 15) ^ fg;            // chunk 2*ks + fg of row krow sits at ((2*(ks%8)) ^ kx) + 16*(ks/8)
+    const unsigned char* kbase = smem + PP_LDS_K + krow * 512;
+    float mrun = -INFINITY;                     // running maximum of s * sc2
+    typename mma<T>::frag kf[KS];
+    auto read_k = [&](int tile, int ks_lo, int ks_hi) {
+      const unsigned char* kp = kbase + (tile & (PP_STAGES - 1)) * PP_KTILE;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        if (ks >= ks_lo && ks < ks_hi)
+          kf[ks] = mma<T>::load(reinterpret_cast<const T*>(kp + (((2 * (ks & 7)) ^ kx) * 16) + (ks >> 3) * 256));
+    };
+    __builtin_amdgcn_s_barrier();               // tile 0 has landed (the value wavefronts waited for it)
+    if (ntiles > 0) read_k(0, 0, 8);
+    for (int i = 0; i <= ntiles; ++i) {
+      const int key0 = i * BKV;
+      const bool active = i < ntiles && key0 <= wave_last;
+      floatx16 s;
+      if (active) {
+        // one accumulation chain (dependent MFMAs of one shape issue back to back); the fragments of k-steps 0-7 were
+        // fetched in the previous phase, those of k-steps 8-15 arrive under the first eight MFMAs
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = 0.f;
+        read_k(i, 8, 16);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) mma<T>::run(s, kf[ks], qf[ks]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_s_barrier();
+      if (active) {
+        // register v is key key0 + 16*(v/8) + 8*fg + v%8
+        if (key0 + BKV - 1 > wave_first) {      // the diagonal crosses the tile: hide what a query may not see
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int key = key0 + 16 * (v / 8) + 8 * fg + (v % 8);
+            s[v] = (key <= qsee) ? s[v] : -INFINITY;
+          }
+        }
+        float mt = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+        for (int v = 3; v < 15; v += 2) mt = fmaxf(fmaxf(mt, s[v]), s[v + 1]);
+        mt = fmaxf(mt, s[15]) * sc2;            // sc2 > 0
+        mt = max_halves(mt);
+        // the running maximum only moves when some lane's tile maximum exceeds it by more than 2^6 (probabilities stay
+        // below 64), so the partner rescales its accumulator in the first tiles only
+        const bool moved = __any(mt > mrun + 6.0f);
+        if (moved) {
+          const float mnew = fmaxf(mrun, mt);
+          *ax = (mnew == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(mrun - mnew);   // mrun = -inf -> 0
+          mrun = mnew;
+          ax[64] = (mrun == -INFINITY) ? 0.f : -mrun;
+        }
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4)
+          *reinterpret_cast<floatx4*>(sx + v4 * 256) = floatx4{s[4 * v4], s[4 * v4 + 1], s[4 * v4 + 2], s[4 * v4 + 3]};
+        if (lane == 0) *fx = moved ? 1 : 0;
+      }
+      // K tile i+1 has landed (the value wavefronts waited for it before the barrier above)
+      if (i + 1 < ntiles && key0 + BKV <= wave_last) read_k(i + 1, 0, 8);
+      __builtin_amdgcn_s_barrier();
+    }
+    return;
+  }
+
+  // ---------------- value wavefront
+  floatx16 o[NBLK];
+#pragma unroll
+  for (int i = 0; i < NBLK; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
+  float lrun = 0.f, mneg = 0.f;
+  __builtin_amdgcn_s_waitcnt(wait_vmcnt(12));               // tile 0 of K and V^T
+  __builtin_amdgcn_s_barrier();
+
+  const int vx = (fr >> 2) & 3;
+  const unsigned char* vbase = smem + PP_LDS_V + fr * 64;
+  const int vpos0 = ((0 + fg) ^ vx) * 16, vpos1 = ((2 + fg) ^ vx) * 16;
+  const int last = ntiles > 0 ? ntiles - 1 : 0;
+  for (int i = 0; i <= ntiles; ++i) {
+    // ---- phase 1: the probabilities of tile i-1 and its V^T fragments
+    const int tk3 = i + 3 < last ? i + 3 : last, tv2 = i + 2 < last ? i + 2 : last;   // the tiles requested in phase 2
+    const int tv = i - 1;
+    const bool active = tv >= 0 && tv * BKV <= wave_last;
+    typename mma<T>::frag pf[2], vf[2][NBLK];
+    if (active) {
+      const unsigned char* vp = vbase + (tv & (PP_STAGES - 1)) * PP_VTILE;
+      // the last tile of a sequence can be partial: what V^T holds beyond the last key must not reach the product
+      // (0 x garbage may be NaN).  Every value wavefront clears all of it before its own reads (LDS operations of one
+      // wavefront stay in order), so no barrier is needed.
+      const int nbad = tv * BKV + BKV - 1 - klast;
+      if (nbad > 0) {
+        uint16_t* vs = reinterpret_cast<uint16_t*>(smem + PP_LDS_V + (tv & (PP_STAGES - 1)) * PP_VTILE);
+        for (int c = lane; c < DH * nbad; c += 64) {
+          const int row = c / nbad, col = BKV - nbad + (c % nbad);
+          vs[row * 32 + (((col >> 3) ^ ((row >> 2) & 3)) * 8) + (col & 7)] = (uint16_t)0;
+        }
+      }
+      float p[16];
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const floatx4 sv = *reinterpret_cast<const floatx4*>(sx + v4 * 256);
+        p[4 * v4] = sv.x; p[4 * v4 + 1] = sv.y; p[4 * v4 + 2] = sv.z; p[4 * v4 + 3] = sv.w;
+      }
+      const int moved = *fx;
+#pragma unroll
+      for (int n = 0; n < NBLK; ++n) vf[0][n] = mma<T>::load(reinterpret_cast<const T*>(vp + n * 2048 + vpos0));
+#pragma unroll
+      for (int n = 0; n < NBLK; ++n) vf[1][n] = mma<T>::load(reinterpret_cast<const T*>(vp + n * 2048 + vpos1));
+      if (moved) {
+        const float alpha = *ax;
+        mneg = ax[64];
+        lrun *= alpha;
+#pragma unroll
+        for (int n = 0; n < NBLK; ++n)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o[n][v] *= alpha;
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) p[v] = __builtin_amdgcn_exp2f(fmaf(p[v], sc2, mneg));   // masked -> exp2(-inf) = 0
+      pf[0] = mma<T>::from_floats(p);
+      pf[1] = mma<T>::from_floats(p + 8);
+      float lt = psum<T>::run(pf[1], psum<T>::run(pf[0], 0.f));
+      lrun += sum_halves(lt);
+    }
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(8));              // K of tile i+1 and V^T of tile i have landed
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase 2: O^T += V^T P^T, and the requests for K tile i+3 and V^T tile i+2 (their stages were last read in
+    // iteration i-1), one per two MFMAs.  (Issued by the score wavefronts instead, whose second phase is the longer
+    // one, the kernel is 5 % slower.)
+    if (active) {
+      mma<T>::run(o[0], vf[0][0], pf[0]); mma<T>::run(o[1], vf[0][1], pf[0]);
+      __builtin_amdgcn_sched_barrier(0); issue_k1(i + 3, tk3, J0{}); __builtin_amdgcn_sched_barrier(0);
+      mma<T>::run(o[2], vf[0][2], pf[0]); mma<T>::run(o[3], vf[0][3], pf[0]);
+      __builtin_amdgcn_sched_barrier(0); issue_k1(i + 3, tk3, J1{}); __builtin_amdgcn_sched_barrier(0);
+      mma<T>::run(o[4], vf[0][4], pf[0]); mma<T>::run(o[5], vf[0][5], pf[0]);
+      __builtin_amdgcn_sched_barrier(0); issue_k1(i + 3, tk3, J2{}); __builtin_amdgcn_sched_barrier(0);
+      mma<T>::run(o[6], vf[0][6], pf[0]); mma<T>::run(o[7], vf[0][7], pf[0]);
+      __builtin_amdgcn_sched_barrier(0); issue_k1(i + 3, tk3, J3{}); __builtin_amdgcn_sched_barrier(0);
+      mma<T>::run(o[0], vf[1][0], pf[1]); mma<T>::run(o[1], vf[1][1], pf[1]);
+      __builtin_amdgcn_sched_barrier(0); issue_v1(i + 2, tv2, J0{}); __builtin_amdgcn_sched_barrier(0);
+      mma<T>::run(o[2], vf[1][2], pf[1]); mma<T>::run(o[3], vf[1][3], pf[1]);
+      __builtin_amdgcn_sched_barrier(0); issue_v1(i + 2, tv2, J1{}); __builtin_amdgcn_sched_barrier(0);
+      mma<T>::run(o[4], vf[1][4], pf[1]); mma<T>::run(o[5], vf[1][5], pf[1]);
+      __builtin_amdgcn_sched_barrier(0); issue_v1(i + 2, tv2, J2{}); __builtin_amdgcn_sched_barrier(0);
+      mma<T>::run(o[6], vf[1][6], pf[1]); mma<T>::run(o[7], vf[1][7], pf[1]);
+      __builtin_amdgcn_sched_barrier(0); issue_v1(i + 2, tv2, J3{}); __builtin_amdgcn_sched_barrier(0);
+    } else {
+      issue_k(i + 3, tk3);
+      issue_v(i + 2, tv2);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));                // the surplus loads land before the LDS is given away
+
+  // ---- write O: register v of block n is head-dim n*32 + 8*(v/4) + 4*fg + v%4 of query t
+  if (t < Tp) {
+    const float inv = (qpos >= 0 && lrun > 0.f) ? 1.0f / lrun : 0.f;
+    T* op = out + ((int64_t)b * Tp + t) * ld_out + (int64_t)h * DH;
+#pragma unroll
+    for (int n = 0; n < NBLK; ++n)
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const int e = n * 32 + 8 * v4 + 4 * fg;
+        uint32x2 pk;
+        pk.x = pack2<T>(o[n][v4 * 4] * inv, o[n][v4 * 4 + 1] * inv);
+        pk.y = pack2<T>(o[n][v4 * 4 + 2] * inv, o[n][v4 * 4 + 3] * inv);
+        *reinterpret_cast<uint32x2*>(op + e) = pk;
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Decode.  Grid (S, H, B): the valid part of a (sequence, head) window is cut into S equal key ranges (the cut
 // follows the position read from device memory, so every workgroup has work whatever the fill), and each
 // 4-wavefront workgroup reduces its range to a partial (max, sum, weighted V).  A wavefront owns every fourth
@@ -544,14 +851,27 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
         (const T*)q, (const T*)k_cache, (const T*)v_t, pos0, (int)H, (int)Tp, (int)Tcap, ldvt, (T*)out, ld_out,      \
         (int)B, (int)nqblk, key_limit);                                                                                       \
   } while (0)
-  if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL(bf16_t, 256, 4, 32);
+#define MTJ_PREFILL_PAIR(T)                                                                                          \
+  do {                                                                                                               \
+    static_assert(PP_LDS_BYTES <= 160 * 1024, "attention tiles do not fit LDS");                                     \
+    static mtj_device_once once;                                                                                     \
+    if (int rc = mtj_allow_lds(once, "mtj_attn_prefill", &attn_prefill_pair_kernel<T>, PP_LDS_BYTES)) return rc;     \
+    const int64_t nqblk = (Tp + 127) / 128;                                                                          \
+    MTJ_REQUIRE(nqblk * H * B < (1ll << 31), MTJ_ELIMIT, "mtj_attn_prefill: too many workgroups");                    \
+    MTJ_REQUIRE(Tcap * 512 < (1ll << 31) && 512 * ldvt < (1ll << 31), MTJ_ELIMIT, "mtj_attn_prefill: window too long"); \
+    attn_prefill_pair_kernel<T><<<(unsigned)(nqblk * H * B), 512, PP_LDS_BYTES, s>>>(                                 \
+        (const T*)q, (const T*)k_cache, (const T*)v_t, pos0, (int)H, (int)Tp, (int)Tcap, ldvt, (T*)out, ld_out,      \
+        (int)B, (int)nqblk, key_limit);                                                                              \
+  } while (0)
+  if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL_PAIR(bf16_t);
   else if (dtype == MTJ_BF16 && dh == 64) MTJ_PREFILL(bf16_t, 64, 8, 64);
-  else if (dtype == MTJ_F16 && dh == 256) MTJ_PREFILL(f16_t, 256, 4, 32);
+  else if (dtype == MTJ_F16 && dh == 256) MTJ_PREFILL_PAIR(f16_t);
   else if (dtype == MTJ_F16 && dh == 64) MTJ_PREFILL(f16_t, 64, 8, 64);
   else if (dtype == MTJ_F32 && dh == 256) MTJ_PREFILL(float, 256, 4, 32);
   else if (dtype == MTJ_F32 && dh == 64) MTJ_PREFILL(float, 64, 4, 32);
   else return mtj_fail(MTJ_EINVAL, "mtj_attn_prefill: unsupported dtype %d / d_head %lld (64 or 256)", dtype, (long long)dh);
 #undef MTJ_PREFILL
+#undef MTJ_PREFILL_PAIR
   return mtj_check_launch("mtj_attn_prefill");
 }
 

@@ -220,6 +220,30 @@ __device__ __forceinline__ floatx4 mtj_merge_partials(const float* __restrict__ 
   return acc * inv;
 }
 
+// Exchange between the two 32-lane halves of a wavefront without going through LDS: after the swap `a` holds the
+// lower half's values in both halves and `b` the upper half's, so op(a, b) is the reduction over lanes l and l ^ 32.
+__device__ __forceinline__ void swap_halves(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float max_halves(float x) {
+  float a = x, b = x;
+  swap_halves(a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float sum_halves(float x) {
+  float a = x, b = x;
+  swap_halves(a, b);
+  return a + b;
+}
+
+// destination of a global -> LDS load (buffer_load ... lds)
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+// s_waitcnt immediates that constrain one counter only (gfx9 encoding: vmcnt [3:0] and [15:14], expcnt [6:4],
+// lgkmcnt [11:8])
+constexpr int wait_vmcnt(int n) { return (n & 0xf) | (((n >> 4) & 3) << 14) | (0x7 << 4) | (0xf << 8); }
+constexpr int wait_lgkmcnt(int n) { return 0xf | (3 << 14) | (0x7 << 4) | ((n & 0xf) << 8); }
+
 // jax.nn.gelu(approximate=True): 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3).
 // 0.5 (1 + tanh(u)) = 1 / (1 + exp(-2u)) = 1 / (1 + 2^(x (k1 + k2 x^2))) with k1 = -2 log2(e) sqrt(2/pi) and
 // k2 = 0.044715 k1: three multiplications, one fma, one addition, v_exp_f32 and v_rcp_f32 (about 1 ulp each).  The

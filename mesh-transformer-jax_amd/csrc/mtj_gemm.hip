@@ -576,13 +576,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
   epilogue<EPI, WAVES_M, WAVES_N, WM, WN>(a, out, acc, smem, m0, n0);
 }
 
-typedef __attribute__((address_space(3))) void* lds_ptr;
-
-// s_waitcnt immediates that constrain one counter only (gfx9 encoding: vmcnt [3:0] and [15:14], expcnt [6:4],
-// lgkmcnt [11:8])
-constexpr int wait_vmcnt(int n) { return (n & 0xf) | (((n >> 4) & 3) << 14) | (0x7 << 4) | (0xf << 8); }
-constexpr int wait_lgkmcnt(int n) { return 0xf | (3 << 14) | (0x7 << 4) | ((n & 0xf) << 8); }
-
 // 16-bit operands, 256x256 workgroup tile, 8 wavefronts of 128x64, K step 64, two LDS stages of 64 KiB,
 // v_mfma_f32_16x16x32 (under the board's power limit it sustains a higher clock than the 32x32x16 form: 1820 against
 // 1570 TFLOP/s in a register-only loop on random float16 data).

@@ -607,7 +607,10 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
   const int wm = wave >> 2, wn = wave & 3;
   const int fr = lane & 15, fq = lane >> 4;
 
-  // tile id: as in gemm_kernel (contiguous tile ranges per XCD, groups of 8 row-tiles)
+  // tile id: contiguous tile ranges per XCD; the 32 workgroups that an XCD runs at a time form 8 x 4 tiles (row-tiles x
+  // column-tiles), or 4 x 8 when the problem has few column-tiles (the out projection: each row panel is then fetched
+  // from memory twice instead of four times, the small weight matrix more often; 1.4 % faster there, 0.9 % slower on
+  // the input projection)
   const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
   const int nblk = tiles_m * tiles_n;
   int pid = blockIdx.x;
@@ -615,7 +618,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
     const int per = nblk / 8;
     if (pid < per * 8) pid = (pid % 8) * per + pid / 8;
   }
-  constexpr int GM = 8;
+  const int GM = tiles_n <= 16 ? 4 : 8;
   const int group = pid / (GM * tiles_n);
   const int first_m = group * GM;
   const int gsz = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;

@@ -593,8 +593,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const gemm_
 // wavefronts multiply while the other four read.  Operands are loaded in four sets per k-tile (A rows / W rows
 // of the first and second half of every wavefront's tile) in the order the clusters consume them, each set into
 // the place of the same set two k-tiles earlier as soon as both groups have read that one; every load is issued
-// nine to ten clusters before its first reader.  Loads for k-tiles beyond the range re-read the last k-tile
-// (the stage they land in is not read again), which keeps the wait counts the same in every k-tile.
+// nine to ten clusters before its first reader.
 template <typename T, int EPI>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
   static_assert(sizeof(T) == 2, "16-bit operands");
@@ -650,18 +649,21 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
   // set 0: A first half, 1: W first half, 2: W second half, 3: A second half
   auto issue = [&](int st, int kt, auto SET_) {
     constexpr int set = decltype(SET_)::value;
-    const int koff = (kt0 + (kt < KT ? kt : KT - 1)) * ROWB;
+    const int koff = (kt0 + kt) * ROWB;
+    // a k-tile beyond the range is requested all the same (the wait counts stay the same in every k-tile) but with an
+    // offset far outside the buffer: such a load fetches nothing and writes zeros into a stage that is not read again
+    const int beyond = kt < KT ? 0 : 0x40000000;
     if constexpr (set == 0 || set == 3) {
       const int r = ra0 + (set == 3 ? 64 : 0);
       unsigned char* d = smem + st * STAGEB + r * ROWB;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr)d, 16, voff_a, koff + (int)((int64_t)r * a.lda * 2), 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr)(d + 128 * ROWB), 16, voff_a,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr)d, 16, voff_a + beyond, koff + (int)((int64_t)r * a.lda * 2), 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr)(d + 128 * ROWB), 16, voff_a + beyond,
                                                koff + (int)((int64_t)(r + 128) * a.lda * 2), 0, 0);
     } else {
       const int r = rb0 + (set == 2 ? 32 : 0);
       unsigned char* d = smem + st * STAGEB + OPB + r * ROWB;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr)d, 16, voff_b, koff + (int)((int64_t)r * a.K * 2), 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr)(d + 128 * ROWB), 16, voff_b,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr)d, 16, voff_b + beyond, koff + (int)((int64_t)r * a.K * 2), 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_ptr)(d + 128 * ROWB), 16, voff_b + beyond,
                                                koff + (int)((int64_t)(r + 128) * a.K * 2), 0, 0);
     }
   };
@@ -984,8 +986,8 @@ int check_common(const void* A, int64_t lda, const void* W, int64_t M, int64_t N
   MTJ_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), MTJ_ELIMIT, "%s: dimension too large", who);
   MTJ_REQUIRE(mtj_aligned16(A) && mtj_aligned16(W) && (lda * esz) % 16 == 0, MTJ_EALIGN,
               "%s: A, W and the row stride of A must be 16-byte aligned", who);
-  MTJ_REQUIRE(256 * lda * esz < (1ll << 31) && 256 * K * esz < (1ll << 31), MTJ_ELIMIT,
-              "%s: a 256-row tile of A or W must span less than 2 GiB", who);
+  MTJ_REQUIRE(256 * lda * esz < (1ll << 30) && 256 * K * esz < (1ll << 30), MTJ_ELIMIT,
+              "%s: a 256-row tile of A or W must span less than 1 GiB", who);
   return MTJ_OK;
 }
 

@@ -399,6 +399,35 @@ def test_gemm_resid_and_store_on_the_256x256_direct_to_lds_kernel(L, dt):
     assert rel_err(out, 0.5 * (ref[:M - 100] - bias.double()) + bias.double()) < 5e-6
 
 
+@pytest.mark.parametrize("K", [64, 128, 192, 320])
+@pytest.mark.parametrize("N,ldo", [(4096, 4096), (4090, 4091)])
+def test_direct_to_lds_kernel_with_few_k_tiles_and_ragged_columns(L, K, N, ldo):
+    """One, two, three and five k-tiles of 64 (the main loop of gemm_dma_kernel handles k-tiles in pairs, requests
+    operands two k-tiles ahead and must not read a tile that was never requested), and a column count / output pitch
+    that is not a multiple of four, which sends the epilogue down its element-wise stores (16 x 16 = 256 tiles of
+    256 x 256 either way, so mtj_gemm dispatches that kernel).  Reference: float64 product on the GPU."""
+    a = abi()
+    g = torch.Generator().manual_seed(K + N)
+    M = 4000                                                   # a ragged last row tile as well
+    A = torch.randn(M, K, generator=g).to(torch.float16).to(DEV)
+    Wh = (torch.randn(K, N, generator=g) * 0.05).to(torch.float16).to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    W = _packed(Wh)
+    ref = A.double() @ Wh.double() + bias.double()
+    x0 = torch.randn(M, ldo, generator=g).to(DEV)
+    x = x0.clone()
+    code = a.dtype_code(torch.float16)
+    a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_RESID, a.ptr(x), ldo, 0, None, 1.0, S()))
+    out = torch.full((M, ldo), 7.0, dtype=torch.float16, device=DEV)
+    a.check(L.mtj_gemm(a.ptr(A), K, a.ptr(W), a.ptr(bias), M, N, K, code, a.EPI_STORE, a.ptr(out), ldo, a.dtype_code(torch.float16),
+                       None, 1.0, S()))
+    torch.cuda.synchronize()
+    assert rel_err(x[:, :N], x0[:, :N].double() + ref) < 5e-6
+    assert torch.equal(x[:, N:], x0[:, N:])                    # nothing written beyond column N
+    assert rel_err(out[:, :N], ref) < 1e-3                     # float16 output
+    assert bool((out[:, N:] == 7.0).all())
+
+
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 def test_inproj_gemv_decode_appends_to_ring(dt):
     from mesh_transformer.engine import Engine

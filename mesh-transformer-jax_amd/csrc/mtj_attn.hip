@@ -28,6 +28,9 @@ template <> struct mma<bf16_t> {
   __device__ static __forceinline__ void run(floatx16& c, const frag& a, const frag& b) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
   }
+  __device__ static __forceinline__ floatx16 first(const frag& a, const frag& b) {   // product alone: C is the constant 0
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, floatx16{}, 0, 0, 0);
+  }
 };
 template <> struct mma<f16_t> {
   static constexpr int EPC = 8;
@@ -48,6 +51,9 @@ template <> struct mma<f16_t> {
   }
   __device__ static __forceinline__ void run(floatx16& c, const frag& a, const frag& b) {
     c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.v, b.v, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ floatx16 first(const frag& a, const frag& b) {   // product alone: C is the constant 0
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a.v, b.v, floatx16{}, 0, 0, 0);
   }
 };
 template <> struct mma<float> {
@@ -434,27 +440,33 @@ __global__ __launch_bounds__(512) void attn_prefill_pair_kernel(const T* __restr
   // position l % 32 of row 2j + l / 32 with chunk (p & 16) | ((p & 15) ^ (row & 15)).  V^T tile: 256 rows x 64 bytes =
   // 16 loads of 16 rows; lane l fills position l % 4 of row 16j + l / 4 with chunk (l % 4) ^ ((row / 4) % 4).
   const int wb = wave & 3;
-  int k_row[4], k_chunk[4], v_off[4];
+  int k_row[4], k_chunk[4], k_off[4], v_off[4];
 #pragma unroll
   for (int jj = 0; jj < 4; ++jj) {
     const int j = 4 * wb + jj;
     k_row[jj] = 2 * j + (lane >> 5);
     const int kp_l = lane & 31;
     k_chunk[jj] = ((kp_l & 16) | ((kp_l & 15) ^ (k_row[jj] & 15))) * 16;
+    k_off[jj] = k_row[jj] * 512 + k_chunk[jj];
     const int vrow_l = 16 * j + (lane >> 2);
     v_off[jj] = (int)((int64_t)vrow_l * ldvt * 2) + (((lane & 3) ^ ((vrow_l >> 2) & 3)) * 16);
   }
   auto issue_k1 = [&](int stage_tile, int tile, auto JJ_) {
     constexpr int jj = decltype(JJ_)::value;
     unsigned char* dst = smem + PP_LDS_K + (stage_tile & (PP_STAGES - 1)) * PP_KTILE + wb * 4096 + jj * 1024;
-    const int row = tile * BKV + k_row[jj];                 // rows beyond the last key are masked by their readers
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)dst, 16, (row < Tcap ? row : Tcap - 1) * 512 + k_chunk[jj], 0, 0, 0);
+    // rows beyond the last key are masked by their readers; rows beyond the window repeat its last row
+    if (tile * BKV + BKV <= Tcap) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)dst, 16, k_off[jj] + tile * (BKV * 512), 0, 0, 0);
+    } else {
+      const int row = tile * BKV + k_row[jj];
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)dst, 16, (row < Tcap ? row : Tcap - 1) * 512 + k_chunk[jj], 0, 0, 0);
+    }
   };
   auto issue_v1 = [&](int stage_tile, int tile, auto JJ_) {
     constexpr int jj = decltype(JJ_)::value;
     unsigned char* dst = smem + PP_LDS_V + (stage_tile & (PP_STAGES - 1)) * PP_VTILE + wb * 4096 + jj * 1024;
-    const int64_t col = (int64_t)tile * BKV + BKV <= ldvt ? (int64_t)tile * BKV : ldvt - BKV;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)dst, 16, v_off[jj] + (int)col * 2, 0, 0, 0);
+    const int col = (int64_t)tile * BKV + BKV <= ldvt ? tile * BKV : (int)ldvt - BKV;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)dst, 16, v_off[jj] + col * 2, 0, 0, 0);
   };
   using J0 = std::integral_constant<int, 0>;
   using J1 = std::integral_constant<int, 1>;
@@ -490,15 +502,16 @@ __global__ __launch_bounds__(512) void attn_prefill_pair_kernel(const T* __restr
     // row fr of an S^T block is key krow: rows {0-3, 4-7, 8-11, 12-15} <- keys {0-3, 8-11, 4-7, 12-15} (+16)
     const int krow = 16 * (fr >> 4) + 8 * ((fr >> 2) & 1) + 4 * ((fr >> 3) & 1) + (fr & 3);
     const int kx = (krow & 15) ^ fg;            // chunk 2*ks + fg of row krow sits at ((2*(ks%8)) ^ kx) + 16*(ks/8)
-    const unsigned char* kbase = smem + PP_LDS_K + krow * 512;
     float mrun = -INFINITY;                     // running maximum of s * sc2
     typename mma<T>::frag kf[KS];
+    int kxo[8];                                 // byte offset of chunk 2*k + fg of my row inside a 256-byte half row
+#pragma unroll
+    for (int k = 0; k < 8; ++k) kxo[k] = krow * 512 + (((2 * k) ^ kx) * 16);
     auto read_k = [&](int tile, int ks_lo, int ks_hi) {
-      const unsigned char* kp = kbase + (tile & (PP_STAGES - 1)) * PP_KTILE;
+      const unsigned char* kp = smem + PP_LDS_K + (tile & (PP_STAGES - 1)) * PP_KTILE;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
-        if (ks >= ks_lo && ks < ks_hi)
-          kf[ks] = mma<T>::load(reinterpret_cast<const T*>(kp + (((2 * (ks & 7)) ^ kx) * 16) + (ks >> 3) * 256));
+        if (ks >= ks_lo && ks < ks_hi) kf[ks] = mma<T>::load(reinterpret_cast<const T*>(kp + kxo[ks & 7] + (ks >> 3) * 256));
     };
     __builtin_amdgcn_s_barrier();               // tile 0 has landed (the value wavefronts waited for it)
     if (ntiles > 0) read_k(0, 0, 8);
@@ -509,12 +522,11 @@ __global__ __launch_bounds__(512) void attn_prefill_pair_kernel(const T* __restr
       if (active) {
         // one accumulation chain (dependent MFMAs of one shape issue back to back); the fragments of k-steps 0-7 were
         // fetched in the previous phase, those of k-steps 8-15 arrive under the first eight MFMAs
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = 0.f;
         read_k(i, 8, 16);
         __builtin_amdgcn_sched_barrier(0);
+        s = mma<T>::first(kf[0], qf[0]);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) mma<T>::run(s, kf[ks], qf[ks]);
+        for (int ks = 1; ks < KS; ++ks) mma<T>::run(s, kf[ks], qf[ks]);
         __builtin_amdgcn_sched_barrier(0);
       }
       __builtin_amdgcn_s_barrier();

@@ -130,7 +130,9 @@ int mtj_xent(const float* logits, int64_t ld, const int32_t* target, int64_t M, 
 /* C = alpha * A[M, K] (dtype, row stride lda) x W[N, K]^T (packed, dtype) with epilogue `epi`.
  * hk.Linear call sites: layers.py:249-258, 559.  MFMA kernel; bias is float32 [N] or NULL; alpha undoes the scale
  * of mtj_pack_weight_cvt (1 otherwise) and multiplies the float32 accumulator before anything else is applied.
- * STORE: out [M, ldo] in out_dtype.  RESID: out float32 [M, ldo].  INPROJ: `ip` non-NULL, bias = b1 [F]. */
+ * STORE: out [M, ldo] in out_dtype.  RESID: out float32 [M, ldo].  INPROJ: `ip` non-NULL, bias = b1 [F].
+ * K must be a multiple of 64 (32 for float32), A, W and the rows of A 16-byte aligned, and 256 rows of A or W must
+ * span less than 1 GiB (MTJ_ELIMIT otherwise). */
 int mtj_gemm(const void* A, int64_t lda, const void* W, const float* bias, int64_t M, int64_t N, int64_t K,
              int dtype, int epi, void* out, int64_t ldo, int out_dtype, const mtj_inproj* ip, float alpha,
              void* stream);

@@ -174,7 +174,7 @@ int mtj_gemm_xent(const void* A, int64_t lda, const void* W, const float* bias, 
  * If ln_scale != NULL the kernel first applies LayerNorm(x) (layers.py:17-36) - x then has K = d entries.
  * If am != NULL (no LayerNorm then) the first am->n_heads * am->d_head entries of the input are not read from x but
  * merged from the attention partials of batch row 0 (mtj_attn_decode_partials).
- * Same epilogues as mtj_gemm with M = 1. */
+ * Same epilogues as mtj_gemm with M = 1; with MTJ_EPI_INPROJ, n_heads * Tcap * d_head, N and ld_act must be below 2^31. */
 int mtj_gemv(const float* x, const float* ln_scale, const float* ln_offset, const void* W, const float* bias,
              int64_t N, int64_t K, int dtype, int epi, void* out, int out_dtype, const mtj_inproj* ip,
              const mtj_attn_merge* am, void* stream);

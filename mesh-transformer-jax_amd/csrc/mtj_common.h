@@ -305,6 +305,54 @@ __device__ __forceinline__ inproj_pre inproj_prepare(const mtj_inproj& ip, const
   return p;
 }
 
+// The same two halves for row 0 of a one-token call (Tp == 1: sequence 0, token 0, no transposed copy of V), as the
+// matrix-vector kernels need them: 32-bit arithmetic, a single division, four registers.  Same values; the
+// destination index must fit 31 bits (n_heads * Tcap * d_head and ld_act below 2^31, which the callers check).
+struct inproj_tok {
+  int kind;        // as inproj_pre
+  float sn, cs;
+  int idx;
+};
+
+__device__ __forceinline__ inproj_tok inproj_prepare_token(const mtj_inproj& ip, const float* __restrict__ b1, int n) {
+  inproj_tok p;
+  p.sn = 0.f; p.cs = 1.f; p.idx = 0;
+  const int d = ip.n_heads * ip.d_head;
+  if (n >= 3 * d) {  // fc_in -> gelu
+    const int c = n - 3 * d;
+    p.kind = 3;
+    p.cs = b1[c];
+    p.idx = d + c;
+    return p;
+  }
+  const int pos = ip.pos0[0];
+  if (pos < 0) { p.kind = -1; return p; }
+  const int seg = (n >= d ? 1 : 0) + (n >= 2 * d ? 1 : 0);   // 0 q, 1 v, 2 k
+  const int c = n - seg * d;
+  const int h = (int)((unsigned)c / (unsigned)ip.d_head), e = c - h * ip.d_head;
+  p.kind = seg;
+  if (seg != 1 && e < ip.rotary_dims) {
+    const int pp = pos < ip.max_pos ? pos : ip.max_pos - 1;
+    const float sn = ip.sin_tab[(int64_t)pp * (ip.rotary_dims / 2) + (e >> 1)];
+    p.cs = ip.cos_tab[(int64_t)pp * (ip.rotary_dims / 2) + (e >> 1)];
+    p.sn = (e & 1) ? sn : -sn;
+  }
+  if (seg == 0) p.idx = c;
+  else p.idx = (h * ip.Tcap + (int)((unsigned)pos % (unsigned)ip.Tcap)) * ip.d_head + e;
+  return p;
+}
+
+__device__ __forceinline__ void inproj_finish_token(const mtj_inproj& ip, const inproj_tok& p, float own, float partner) {
+  if (p.kind < 0) return;
+  if (p.kind == 3) {
+    store_as(ip.act, p.idx, gelu_tanh(own + p.cs), ip.act_dtype);
+    return;
+  }
+  const float val = own * p.cs + partner * p.sn;
+  if (p.kind == 0) store_as(ip.q, p.idx, val, ip.q_dtype);
+  else store_as(p.kind == 1 ? ip.v_cache : ip.k_cache, p.idx, val, ip.kv_dtype);
+}
+
 __device__ __forceinline__ void inproj_finish(const mtj_inproj& ip, const inproj_pre& p, float own, float partner) {
   const int kv_dtype = ip.kv_dtype;
   if (p.kind < 0) return;

@@ -59,78 +59,19 @@ struct gemv_args {
   int out_dtype;
   mtj_inproj ip;
   mtj_attn_merge am;      // partials == NULL: x is read as it is
+  int upb, upb_rem;       // units per workgroup: the first upb_rem workgroups take upb + 1 (set by launch())
 };
 
-// One workgroup of 16 wavefronts per CU, all resident at once (a second round of workgroups would pay the
-// prologue and the drain of the memory pipeline twice).  The rows (row pairs for the fused input projection,
-// whose rotary epilogue needs both halves of a pair) are dealt out in equal contiguous ranges over all
-// wavefronts of the grid.  Nothing on the streaming path depends on a second global load: x is requested
-// first, then the first U KiB of weights (so the LayerNorm prologue overlaps the first HBM round trip), and
-// every epilogue operand (position, sin/cos, biases, the residual) is fetched up front by the lane that
-// will finish that row - under load a dependent load costs tens of microseconds.
-//
-// FULL: K is a whole number of wavefront tiles (U x 64 lanes x 16 bytes).  The rows of a wavefront are then one
-// contiguous run of whole tiles, which is streamed with two tiles in flight - the next one is requested before the
-// current one is consumed, so a wavefront never has an empty memory queue - and no load is conditional.  (Dealing
-// the rows out round-robin instead, so that the chip reads one contiguous window at a time, streams ~5 % faster in
-// a plain read but not here: 43.5 us against 40.2 for the 235 MB launch with every lane's epilogue scattered, 40.9
-// against 39.4 with the row sums routed through LDS so that one thread finishes a row and adjacent threads adjacent
-// rows; cutting the rows into 1 KiB pieces so that consecutive wavefronts read consecutive KiB takes 49.7 us.)
-// MERGE: the leading inputs are merged from one-token attention partials (a.am) instead of being read from x.
-template <typename T, int U, bool FULL, bool MERGE>
-__global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
-  extern __shared__ __align__(16) float xs[];
-  __shared__ float red[2][16];
-  constexpr int EPC = chunk<T>::EPC;
-  constexpr int STEP = 64 * EPC;  // elements one wavefront covers per load
+// Stages the input vector of a matrix-vector kernel into LDS: LayerNorm on the fly (two passes, as the reference
+// computes jnp.var), or the attention partials merged into the leading H * dh entries (MERGE), or a plain copy.
+// xv holds this thread's four values when fast_x (K == 4 * blockDim.x, requested by the caller before anything else).
+// Ends with a workgroup barrier.
+template <bool MERGE>
+__device__ __forceinline__ void stage_x(const gemv_args& a, float* __restrict__ xs, float (&red)[2][16], const floatx4& xv,
+                                        bool fast_x) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
   const int K = (int)a.K;
-  const T* __restrict__ W = reinterpret_cast<const T*>(a.W);
-
-  const bool pairs = a.epi == MTJ_EPI_INPROJ;
-  const int64_t upw = pairs ? 2 : 1;
-  const int64_t units = a.N / upw;
-  // The units of a workgroup (an equal contiguous share of all) go to its wavefronts in contiguous runs, the odd
-  // ones to the FIRST wavefronts: under a saturated memory system the wavefronts of a SIMD are served oldest
-  // first and the youngest finish last, so they should be the ones with less to do.
-  const int64_t ub0 = units * blockIdx.x / gridDim.x, ub1 = units * (blockIdx.x + 1) / gridDim.x;
-  const int cnt = (int)(ub1 - ub0), per = cnt / nwaves, rem = cnt % nwaves;
-  const int64_t row0 = (ub0 + (int64_t)wave * per + (wave < rem ? wave : rem)) * upw;
-  const int nrows = (per + (wave < rem ? 1 : 0)) * (int)upw;   // <= 64 (the host sizes the grid for that)
-
-  // ---- x first (4 values per thread while K <= 4096; the general loop below covers the rest) ...
   const bool ln = a.ln_scale != nullptr;
-  floatx4 xv = {0.f, 0.f, 0.f, 0.f};
-  const bool fast_x = ln && K == 4 * (int)blockDim.x;
-  if (fast_x) xv = *reinterpret_cast<const floatx4*>(a.x + 4 * tid);
-  // ---- ... then the epilogue operands of "my" row (lane j finishes row row0 + j) ...
-  inproj_pre pre;
-  pre.kind = -1;
-  float pre_add = 0.f;
-  if (lane < nrows) {
-    const int64_t n = row0 + lane;
-    if (pairs) pre = inproj_prepare(a.ip, a.bias, 0, n);
-    else {
-      pre_add = a.bias ? a.bias[n] : 0.f;
-      if (a.epi == MTJ_EPI_RESID) pre_add += reinterpret_cast<const float*>(a.out)[n];
-    }
-  }
-  // ---- ... then the first tile of weights
-  uint32x4 w[U];
-  if (FULL) {
-    const T* rowp = W + (nrows > 0 ? row0 : 0) * a.K;      // a wavefront without rows reads (and drops) row 0
-#pragma unroll
-    for (int u = 0; u < U; ++u) w[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(rowp + u * STEP + lane * EPC));
-  } else if (nrows > 0) {
-    const T* rowp = W + row0 * a.K;
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int k = u * STEP + lane * EPC;
-      if (k < K) w[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(rowp + k));
-    }
-  }
-
-  // ---- stage x (with LayerNorm if asked) into LDS
   if (ln) {
     float s = 0.f;
     if (fast_x) {
@@ -187,14 +128,92 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   }
   __syncthreads();
 
-  // ---- stream my rows; lane r keeps the sum of row r
+}
+
+// One workgroup of 16 wavefronts per CU, all resident at once (a second round of workgroups would pay the
+// prologue and the drain of the memory pipeline twice).  The rows (row pairs for the fused input projection,
+// whose rotary epilogue needs both halves of a pair) are dealt out in equal contiguous ranges over all
+// wavefronts of the grid.  Nothing on the streaming path depends on a second global load: x is requested
+// first, then the first U KiB of weights (so the LayerNorm prologue overlaps the first HBM round trip), and
+// every epilogue operand (position, sin/cos, biases, the residual) is fetched up front by the lane that
+// will finish that row - under load a dependent load costs tens of microseconds.
+//
+// FULL: K is a whole number of wavefront tiles (U x 64 lanes x 16 bytes).  The rows of a wavefront are then one
+// contiguous run of whole tiles, which is streamed with two tiles in flight - the next one is requested before the
+// current one is consumed, so a wavefront never has an empty memory queue - and no load is conditional.  (Dealing
+// the rows out round-robin instead, so that the chip reads one contiguous window at a time, streams ~5 % faster in
+// a plain read but not here: 43.5 us against 40.2 for the 235 MB launch with every lane's epilogue scattered, 40.9
+// against 39.4 with the row sums routed through LDS so that one thread finishes a row and adjacent threads adjacent
+// rows; cutting the rows into 1 KiB pieces so that consecutive wavefronts read consecutive KiB takes 49.7 us.)
+// MERGE: the leading inputs are merged from one-token attention partials (a.am) instead of being read from x.
+template <typename T, int U, bool FULL, bool MERGE>
+__global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
+  extern __shared__ __align__(16) float xs[];
+  __shared__ float red[2][16];
+  constexpr int EPC = chunk<T>::EPC;
+  constexpr int STEP = 64 * EPC;  // elements one wavefront covers per load
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int K = (int)a.K;
+  const T* __restrict__ W = reinterpret_cast<const T*>(a.W);
+
+  const bool pairs = a.epi == MTJ_EPI_INPROJ;
+  const int upw = pairs ? 2 : 1;
+  // The units of a workgroup (an equal contiguous share of all, cut on the host: no division stands between the
+  // start of a wavefront and its first request) go to its sixteen wavefronts in contiguous runs, the odd ones to the
+  // FIRST wavefronts: under a saturated memory system the wavefronts of a SIMD are served oldest first and the
+  // youngest finish last, so they should be the ones with less to do.
+  const int bx = blockIdx.x;
+  const int ub0 = bx * a.upb + (bx < a.upb_rem ? bx : a.upb_rem);
+  const int cnt = a.upb + (bx < a.upb_rem ? 1 : 0), per = cnt >> 4, rem = cnt & 15;
+  const int64_t row0 = (int64_t)(ub0 + wave * per + (wave < rem ? wave : rem)) * upw;
+  const int nrows = (per + (wave < rem ? 1 : 0)) * upw;       // <= 64 (the host sizes the grid for that)
+
+  // ---- x first (4 values per thread while K <= 4096; the general loop below covers the rest) ...
+  const bool ln = a.ln_scale != nullptr;
+  floatx4 xv = {0.f, 0.f, 0.f, 0.f};
+  const bool fast_x = ln && K == 4 * (int)blockDim.x;
+  if (fast_x) xv = *reinterpret_cast<const floatx4*>(a.x + 4 * tid);
+  // ---- ... then the first tile of weights: everything else a wavefront has to work out happens while it is on
+  // its way.  (One tile: the CU's memory pipeline takes about 100 KB of requests; the youngest wavefronts already
+  // wait 3 us to place theirs, and the LayerNorm's barriers wait for them.  With two tiles per wavefront requested
+  // up front they wait 6 us and the launch takes 43 us instead of 39.)
   const int tpr = (K + STEP * U - 1) / (STEP * U);          // tiles per row
+  uint32x4 w[U], w2[U];
+  __builtin_amdgcn_sched_barrier(0);
+  if (FULL) {
+    const T* rowp = W + (nrows > 0 ? row0 : 0) * a.K;      // a wavefront without rows reads (and drops) row 0
+#pragma unroll
+    for (int u = 0; u < U; ++u) w[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(rowp + u * STEP + lane * EPC));
+  } else if (nrows > 0) {
+    const T* rowp = W + row0 * a.K;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = u * STEP + lane * EPC;
+      if (k < K) w[u] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(rowp + k));
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // ---- ... then the epilogue operands of "my" row (lane j finishes row row0 + j)
+  inproj_tok pre;
+  pre.kind = -1;
+  float pre_add = 0.f;
+  if (lane < nrows) {
+    const int64_t n = row0 + lane;
+    if (pairs) pre = inproj_prepare_token(a.ip, a.bias, (int)n);
+    else {
+      pre_add = a.bias ? a.bias[n] : 0.f;
+      if (a.epi == MTJ_EPI_RESID) pre_add += reinterpret_cast<const float*>(a.out)[n];
+    }
+  }
+
+  stage_x<MERGE>(a, xs, red, xv, fast_x);
+
+  // ---- stream my rows; lane r keeps the sum of row r
   float mine = 0.f;
   if (FULL) {
     constexpr int TILE = STEP * U;
     const T* base = W + row0 * a.K + lane * EPC;            // tile g of this wavefront starts at base + g * TILE
     const int ntiles = nrows * tpr;
-    uint32x4 w2[U];
     float acc = 0.f;
     int kt = 0, r = 0;
     auto consume = [&](const uint32x4 (&t)[U]) {
@@ -253,7 +272,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   // ---- epilogue: every lane finishes its own row
   if (pairs) {
     const float partner = __shfl_xor(mine, 1);
-    if (lane < nrows) inproj_finish(a.ip, pre, mine, partner);
+    if (lane < nrows) inproj_finish_token(a.ip, pre, mine, partner);
   } else if (lane < nrows) {
     const int64_t n = row0 + lane;
     if (a.epi == MTJ_EPI_STORE) store_as(a.out, n, mine + pre_add, a.out_dtype);
@@ -272,7 +291,10 @@ int launch(const gemv_args& a, hipStream_t s) {
   while ((units + grid * 16 - 1) / (grid * 16) * upw > 62) grid *= 2;   // a lane per row: <= 64 rows per wavefront
   static mtj_device_once once;
   if (int rc = mtj_allow_lds(once, "mtj_gemv", &gemv_kernel<T, U, FULL, MERGE>, 160 * 1024 - 256)) return rc;
-  gemv_kernel<T, U, FULL, MERGE><<<(unsigned)grid, 1024, lds, s>>>(a);
+  gemv_args b = a;
+  b.upb = (int)(units / grid);
+  b.upb_rem = (int)(units % grid);
+  gemv_kernel<T, U, FULL, MERGE><<<(unsigned)grid, 1024, lds, s>>>(b);
   return mtj_check_launch("mtj_gemv");
 }
 
@@ -330,9 +352,10 @@ __global__ __launch_bounds__(1024) void gemv_outatt_kernel(const outatt_args oa)
   const int nwg = gridDim.x;
 
   // rows of this wavefront: as in gemv_kernel
-  const int64_t ub0 = a.N * blockIdx.x / nwg, ub1 = a.N * (blockIdx.x + 1) / nwg;
-  const int cnt = (int)(ub1 - ub0), per = cnt / 16, rem = cnt % 16;
-  const int64_t row0 = ub0 + (int64_t)wave * per + (wave < rem ? wave : rem);
+  const int bx = blockIdx.x;
+  const int ub0 = bx * a.upb + (bx < a.upb_rem ? bx : a.upb_rem);
+  const int cnt = a.upb + (bx < a.upb_rem ? 1 : 0), per = cnt >> 4, rem = cnt & 15;
+  const int64_t row0 = ub0 + wave * per + (wave < rem ? wave : rem);
   const int nrows = per + (wave < rem ? 1 : 0);
 
   const int p = oa.pos[0];
@@ -581,6 +604,8 @@ extern "C" int mtj_gemv(const float* x, const float* ln_scale, const float* ln_o
     MTJ_REQUIRE(ip && bias, MTJ_EINVAL, "mtj_gemv: INPROJ needs ip and the fc_in bias");
     a.ip = *ip;
     const int64_t d = (int64_t)ip->n_heads * ip->d_head;
+    MTJ_REQUIRE((int64_t)ip->n_heads * ip->Tcap * ip->d_head < (1ll << 31) && N < (1ll << 31) && ip->ld_act < (1ll << 31), MTJ_ELIMIT,
+                "mtj_gemv: n_heads * Tcap * d_head, N and ld_act must be below 2^31");
     MTJ_REQUIRE(ip->Tp == 1 && N > 3 * d && N % 2 == 0 && ip->rotary_dims % 2 == 0 && ip->rotary_dims <= ip->d_head &&
                     ip->Tcap > 0 && ip->max_pos > 0 && ip->pos0 && ip->sin_tab && ip->cos_tab && ip->q && ip->k_cache &&
                     ip->v_cache && ip->act && ip->ld_act >= N - 2 * d &&
@@ -682,6 +707,7 @@ extern "C" int mtj_gemv_attn(const float* x, const void* W, const float* bias, i
   outatt_args oa{};
   oa.g.x = x; oa.g.W = W; oa.g.bias = bias; oa.g.N = N; oa.g.K = K; oa.g.epi = MTJ_EPI_RESID; oa.g.out = out;
   oa.g.out_dtype = MTJ_F32;
+  oa.g.upb = (int)(N / plan.grid); oa.g.upb_rem = (int)(N % plan.grid);
   oa.q = q; oa.kc = k_cache; oa.vc = v_cache; oa.pos = pos; oa.H = (int)H; oa.Tcap = (int)Tcap; oa.S = plan.S;
   oa.work = reinterpret_cast<float*>(work);
   hipStream_t s = (hipStream_t)stream;

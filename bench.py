@@ -33,7 +33,7 @@ for p in (ROOT, os.path.join(ROOT, "mesh-transformer-jax_amd")):
 HBM_PEAK = 8.0e12          # B/s
 # HBM bytes of one launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what
 # the same counter reads for a plain 234,881,024-byte copy (profiles/gemv_inproj_hbm_traffic_pmc.md)
-DOMINANT_KERNEL_TRAFFIC = 236080000
+DOMINANT_KERNEL_TRAFFIC = 235603535
 MFMA_BF16_PEAK = 2.5e15    # flop/s dense
 
 CFG_6B = dict(layers=28, d_model=4096, n_heads=16, n_vocab=50400, norm="layernorm", pe="rotary", pe_rotary_dims=64,

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define MTJ_ABI_VERSION 2
+#define MTJ_ABI_VERSION 3
 
 enum { MTJ_F32 = 0, MTJ_BF16 = 1, MTJ_F16 = 2 };
 
@@ -120,6 +120,14 @@ int mtj_embed(const int32_t* tok, int64_t M, const void* W, const float* b, int6
 int mtj_layernorm(const float* x, const float* scale, const float* offset, int64_t M, int64_t d,
                   void* out, int out_dtype, void* stream);
 
+/* Rotary position embedding of projected q / k rows and the K/V window append, without the projection
+ * (fixed_pos_embedding + apply_rotary_pos_emb inside self_attn, layers.py:128-148, 261-273; the window update of
+ * decode_once, layers.py:325-326).  q, v, k float32 [M, H*dh] (any may be NULL and is then skipped); row m is token
+ * m % Tp of sequence m / Tp at position pos0[b] + t, and goes where the fused input projection (MTJ_EPI_INPROJ) puts
+ * it: q rotated into ip->q, k rotated into ip->k_cache, v into ip->v_cache (and ip->v_t when given); ip->act is not
+ * used.  The module-level self_attn of the Python surface is built on it. */
+int mtj_rope_append(const float* q, const float* v, const float* k, int64_t M, const mtj_inproj* ip, void* stream);
+
 /* Per-row cross entropy of float32 logits [M, V] (row stride ld) against int32 targets [M]:
  * ProjectionShard.loss, layers.py:569-593, on one shard: loss = log(sum exp(l - max)) - (l[target] - max),
  * correct = (l[target] == max).  A target outside [0, V) selects nothing (loss = log-sum-exp), like an all-zero
@@ -190,8 +198,10 @@ int mtj_gemv(const float* x, const float* ln_scale, const float* ln_offset, cons
  * x float32 [K] (its first H*dh entries are not read); q float32 [H, dh]; caches [H, Tcap, dh] in kv_dtype; pos
  * int32 [1].  `work`: mtj_gemv_attn_work_bytes(H, dh) bytes, 128-byte aligned, zeroed by the caller ONCE before its
  * first use and then left alone (it holds a running arrival counter); launches sharing one `work` must not overlap
- * and must all have the same N.  Word 2 of `work` becomes non-zero if a launch ever gave up waiting (its result is
- * then unusable). */
+ * and must all have the same N.  The wait is bounded by real time (5 ms of the device's 100 MHz counter): a launch
+ * whose workgroups are not all resident within that time (CUs masked off or held by other work) gives up and sets
+ * word 2 (uint32) of `work`; its result and that of every later launch is then unusable, and later launches no
+ * longer wait, until the caller has written 0 to that word (the arrival counter in words 0-1 must be left alone). */
 int mtj_gemv_attn_supported(int64_t N, int64_t K, int dtype, int64_t H, int64_t dh, int kv_dtype, int64_t Tcap);
 int64_t mtj_gemv_attn_work_bytes(int64_t H, int64_t dh);
 int mtj_gemv_attn(const float* x, const void* W, const float* bias, int64_t N, int64_t K, int dtype, float* out,

@@ -209,6 +209,40 @@ extern "C" int mtj_layernorm(const float* x, const float* scale, const float* of
   return mtj_check_launch("mtj_layernorm");
 }
 
+// ---------------------------------------------------------------- rotary embedding + K/V window append on its own
+// The epilogue of the fused input projection applied to rows that are already projected: element (m, c) of q, v, k
+// [M, d] goes where inproj_store sends column c, d + c, 2d + c of row m (layers.py:261-273: interleaved rotation of
+// the first rotary_dims of every head of q and k at position pos0[b] + t; layers.py:325-326: the window slot).
+__global__ __launch_bounds__(256) void rope_append_kernel(const float* __restrict__ q, const float* __restrict__ v,
+                                                          const float* __restrict__ k, int64_t M, const mtj_inproj ip) {
+  const int d = ip.n_heads * ip.d_head;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= M * d) return;
+  const int64_t m = i / d;
+  const int c = (int)(i - m * d);
+  const float* src[3] = {q, v, k};
+#pragma unroll
+  for (int seg = 0; seg < 3; ++seg) {
+    if (!src[seg]) continue;
+    inproj_store(ip, nullptr, m, (int64_t)seg * d + c, src[seg][m * d + c], src[seg][m * d + (c ^ 1)]);
+  }
+}
+
+extern "C" int mtj_rope_append(const float* q, const float* v, const float* k, int64_t M, const mtj_inproj* ip, void* stream) {
+  MTJ_REQUIRE(ip && M > 0 && (q || v || k), MTJ_EINVAL, "mtj_rope_append: nothing to do");
+  MTJ_REQUIRE(ip->n_heads > 0 && ip->d_head > 0 && ip->d_head % 2 == 0 && ip->rotary_dims % 2 == 0 &&
+                  ip->rotary_dims >= 0 && ip->rotary_dims <= ip->d_head && ip->Tp > 0 && M % ip->Tp == 0 && ip->Tcap > 0 &&
+                  ip->max_pos > 0 && ip->pos0 && ip->sin_tab && ip->cos_tab,
+              MTJ_EINVAL, "mtj_rope_append: inconsistent geometry");
+  MTJ_REQUIRE((!q || (ip->q && mtj_is_dtype(ip->q_dtype))) && (!v || ip->v_cache) && (!k || ip->k_cache) &&
+                  ((!v && !k) || mtj_is_dtype(ip->kv_dtype)) && (!ip->v_t || ip->ldvt >= ip->Tp),
+              MTJ_EINVAL, "mtj_rope_append: a destination is missing for a given source");
+  const int64_t n = M * ip->n_heads * ip->d_head;
+  MTJ_REQUIRE(n < (1ll << 39), MTJ_ELIMIT, "mtj_rope_append: too many elements");
+  rope_append_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(q, v, k, M, *ip);
+  return mtj_check_launch("mtj_rope_append");
+}
+
 // ---------------------------------------------------------------- cross entropy of a logits row
 // ProjectionShard.loss (layers.py:569-593) on one shard: logits -= max; loss = log(sum exp) - logits[target];
 // correct = (logits[target] == 0), i.e. the target holds the row maximum.  One 256-thread workgroup per row.

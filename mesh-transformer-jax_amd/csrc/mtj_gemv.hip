@@ -315,12 +315,14 @@ int launch(const gemv_args& a, hipStream_t s) {
 // of the first pass; exposed are the merge (two batches of four partials, ~2.8 us) and the pipeline drain.
 //
 // The wait needs every workgroup of the grid to be resident at once: the host launches at most one workgroup per
-// CU.  The spin is bounded; if it ever gave up, word 2 of the counter block is set and the result is unusable.
+// CU.  The wait is bounded by real time (5 ms); if it ever gave up, word 2 of the counter block is set, the result is
+// unusable, and every later launch skips its wait until the caller has cleared that word.
 // Counter block: work[0] 64-bit arrival counter (never reset: a launch's target is the next multiple of the grid
 // size above the value its own arrival returned; the caller zeroes `work` once), then the partials, one per
 // (head, range), each in its own 128-byte lines so that no line is shared between writers of different L2s.
 constexpr int OA_NI = 4;              // K (and V) loads per lane and attention step: 128 keys of d_head 256 per workgroup
 constexpr int OA_HEAD = 32;           // floats in front of the partials (counter block)
+constexpr uint64_t OA_WAIT_TICKS = 500000;   // longest wait for the partials: 5 ms of the 100 MHz real-time counter
 
 struct outatt_args {
   gemv_args g;                         // x (entries [0, H*dh) unused), W, bias, N, K, out (residual, in place)
@@ -333,6 +335,48 @@ struct outatt_args {
 };
 
 __device__ __forceinline__ int oa_pstride(int dh) { return (dh + MTJ_DEC_PAD + 31) / 32 * 32; }
+
+// mtj_merge_partials for partials that other workgroups of the SAME launch have written: every load carries sc1, the
+// cache policy of an agent-scope atomic load, so it is served from the level all XCDs share and never from a line this
+// XCD's L2 (or this CU's vector cache) may still hold from an earlier launch - the partials live at the same addresses in
+// every launch.  rs covers the partials (everything behind the counter block), hoff is the byte offset of the head's
+// first partial in it.  Same arithmetic, same order as mtj_merge_partials.
+constexpr int OA_SC1 = 16;            // cache-policy operand of a buffer load: bit 4 = sc1
+__device__ __forceinline__ floatx4 oa_merge_coherent(__amdgpu_buffer_rsrc_t rs, int hoff, int S, int stride, int e) {
+  float mm = -INFINITY, lt = 0.f;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s0 = 0; s0 < S; s0 += 4) {
+    float m[4], l[4];
+    floatx4 v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int off = hoff + (s0 + i < S ? s0 + i : S - 1) * stride * 4;
+      const uint32x2 st = __builtin_bit_cast(uint32x2, __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, OA_SC1));
+      m[i] = __uint_as_float(st.x);
+      l[i] = __uint_as_float(st.y);
+      v[i] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rs, off + (MTJ_DEC_PAD + e) * 4, 0, OA_SC1));
+    }
+    float mb = mm;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (s0 + i >= S) m[i] = -INFINITY;
+      mb = fmaxf(mb, m[i]);
+    }
+    if (mb == -INFINITY) continue;
+    const float r = (mm == -INFINITY) ? 0.f : __expf(mm - mb);
+    lt *= r;
+    acc *= r;
+    mm = mb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float f = (m[i] == -INFINITY) ? 0.f : __expf(m[i] - mm);
+      lt = fmaf(f, l[i], lt);
+      acc += f * v[i];
+    }
+  }
+  const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+  return acc * inv;
+}
 
 template <typename T, typename TKV, int DH>
 __global__ __launch_bounds__(1024) void gemv_outatt_kernel(const outatt_args oa) {
@@ -553,22 +597,35 @@ __global__ __launch_bounds__(1024) void gemv_outatt_kernel(const outatt_args oa)
   // ---- second pass: the attention columns.  Their first tile is requested before the wait.
   if (n2 > 0) request(w, 0, 0, ta);
   if (tid == 0) {
+    // Bounded by real time (the 100 MHz counter): a launch whose workgroups are not all resident - CUs masked off, or
+    // held by another stream for longer than this - ends after OA_WAIT_TICKS, flagged (word 2 of the counter block),
+    // instead of hanging.  Once the flag is up no launch waits any more, so a queue of launches drains at once instead
+    // of timing out one by one; the results are void until the caller has cleared the flag.
     const unsigned long long* cnt = reinterpret_cast<const unsigned long long*>(oa.work);
+    unsigned* flag = reinterpret_cast<unsigned*>(oa.work) + 2;
     const unsigned long long target = (arrived_at / (unsigned)nwg + 1) * (unsigned)nwg;
-    unsigned spins = 0;
+    const uint64_t t0 = __builtin_amdgcn_s_memrealtime();
     while (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
       __builtin_amdgcn_s_sleep(8);
-      if (++spins > (1u << 24)) {                              // some workgroup never arrived: give up, flag it
-        reinterpret_cast<unsigned*>(oa.work)[2] = 1u;
+      if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) break;
+      if (__builtin_amdgcn_s_memrealtime() - t0 > OA_WAIT_TICKS) {   // some workgroup never arrived: give up, flag it
+        __hip_atomic_store(flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         break;
       }
     }
   }
   __syncthreads();
-  for (int k = tid * 4; k < dm; k += 4096) {
-    const int hh = k / DH, e = k - hh * DH;
-    *reinterpret_cast<floatx4*>(xs + k) =
-        mtj_merge_partials(oa.work + OA_HEAD + (int64_t)hh * S * oa_pstride(DH), S, oa_pstride(DH), e);
+  {
+    // The partials were written by other workgroups of this launch with agent-scope stores that had completed
+    // (s_waitcnt) before their writers' arrivals were counted, and the count was seen complete before this point, so
+    // they are at the level the XCDs share; the loads carry sc1 so that they are served from there.
+    const int ps = oa_pstride(DH);
+    const __amdgpu_buffer_rsrc_t prs =
+        __builtin_amdgcn_make_buffer_rsrc(oa.work + OA_HEAD, 0, oa.H * S * ps * 4, 0x00020000);
+    for (int k = tid * 4; k < dm; k += 4096) {
+      const int hh = k / DH, e = k - hh * DH;
+      *reinterpret_cast<floatx4*>(xs + k) = oa_merge_coherent(prs, hh * S * ps * 4, S, ps, e);
+    }
   }
   __syncthreads();
   ct = 0; cr = 0;

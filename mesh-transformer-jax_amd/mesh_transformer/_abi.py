@@ -9,7 +9,7 @@ import os
 
 F32, BF16, F16 = 0, 1, 2
 EPI_STORE, EPI_RESID, EPI_INPROJ = 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmtj_hip.so")
 
@@ -46,6 +46,7 @@ SIGNATURES = {
     "mtj_pack_weight_cvt": (_i32, [_p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _i32, _i32, C.c_float, _p]),
     "mtj_embed": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i32, _p, _p]),
     "mtj_layernorm": (_i32, [_p, _p, _p, _i64, _i64, _p, _i32, _p]),
+    "mtj_rope_append": (_i32, [_p, _p, _p, _i64, C.POINTER(InProj), _p]),
     "mtj_xent": (_i32, [_p, _i64, _p, _i64, _i64, _p, _p, _p]),
     "mtj_gemm": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i32, _i32, _p, _i64, _i32, C.POINTER(InProj), C.c_float, _p]),
     "mtj_gemm_splitk_work_bytes": (_i64, [_i64, _i64, _i64, _i32]),

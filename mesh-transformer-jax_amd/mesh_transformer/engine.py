@@ -310,11 +310,12 @@ class Engine:
         ne.w, ne.bias, ne.x_next, ne.d, ne.dtype = ptr(w.we), ptr(w.be), ptr(ses.x), w.d, w.dtype
         return C.byref(ne)
 
-    def decode_model(self, ses):
-        """generate_once (transformer_shard.py:97-115) from the embedded token in ses.x to the logits; the K/V
-        window is updated in place."""
+    def decode_model(self, ses, logits=None):
+        """generate_once (transformer_shard.py:97-115) from the embedded token in ses.x to the logits (ses.logits, or
+        the [B, V] float32 tensor given); the K/V window is updated in place."""
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()
         B, d, F, V = ses.B, w.d, w.F, w.V
+        logits = ses.logits if logits is None else logits
         if not ses.gemv_path and w.w_p is not None:
             # batched decode: the reduce of every out projection also applies the LayerNorm that follows it (the
             # next layer's, at the end the projection's), so only the first layer launches a LayerNorm of its own
@@ -323,17 +324,17 @@ class Engine:
             for j, i in enumerate(ids):
                 nxt = (w.ln_s[ids[j + 1]], w.ln_o[ids[j + 1]]) if j + 1 < len(ids) else (w.pln_s, w.pln_o)
                 self.layer_decode(ses, i, normed=True, next_ln=nxt)
-            check(L.mtj_gemm(ptr(ses.h), d, ptr(w.w_p_mm), ptr(w.b_p), B, V, d, w.mm_dtype, EPI_STORE, ptr(ses.logits), V,
+            check(L.mtj_gemm(ptr(ses.h), d, ptr(w.w_p_mm), ptr(w.b_p), B, V, d, w.mm_dtype, EPI_STORE, ptr(logits), V,
                              F32, None, w.alpha_p, s))
             return
         for i in w.layer_ids:
             self.layer_decode(ses, i)
         if ses.gemv_path:
             check(L.mtj_gemv(ptr(ses.x), ptr(w.pln_s), ptr(w.pln_o), ptr(w.w_p), ptr(w.b_p), V, d, w.dtype, EPI_STORE,
-                             ptr(ses.logits), F32, None, None, s))
+                             ptr(logits), F32, None, None, s))
         else:
             check(L.mtj_layernorm(ptr(ses.x), ptr(w.pln_s), ptr(w.pln_o), B, d, ptr(ses.h), w.act_dtype, s))
-            check(L.mtj_gemm(ptr(ses.h), d, ptr(w.w_p_mm), ptr(w.b_p), B, V, d, w.mm_dtype, EPI_STORE, ptr(ses.logits), V,
+            check(L.mtj_gemm(ptr(ses.h), d, ptr(w.w_p_mm), ptr(w.b_p), B, V, d, w.mm_dtype, EPI_STORE, ptr(logits), V,
                              F32, None, w.alpha_p, s))
 
     def layer_decode(self, ses, i, normed=False, next_ln=None):
@@ -374,17 +375,17 @@ class Engine:
                                         EPI_RESID, ptr(ses.x), d, F32, ptr(ses.gemm_work), ses.gemm_work.numel(),
                                         w.alpha_out[i], s))
 
-    def sample_greedy(self, ses, out_tokens, embed_next=True):
-        check(_abi.lib().mtj_sample_greedy(ptr(ses.logits), ses.B, self.w.V, ptr(ses.tok), ptr(out_tokens),
+    def sample_greedy(self, ses, out_tokens, embed_next=True, logits=None):
+        check(_abi.lib().mtj_sample_greedy(ptr(ses.logits if logits is None else logits), ses.B, self.w.V, ptr(ses.tok), ptr(out_tokens),
                                            out_tokens.shape[1], ptr(ses.pos), ptr(ses.pos_start),
                                            self._next(ses, embed_next), _abi.stream_handle()))
 
     def sample_nucleus(self, ses, out_tokens, top_p, temp, top_k, uniforms, keep_mask=None, filtered=None,
-                       embed_next=True):
+                       embed_next=True, logits=None):
         L = _abi.lib()
         if ses.sample_work is None:
             ses.sample_work = torch.empty(L.mtj_sample_work_bytes(ses.B, self.w.V), dtype=torch.uint8, device=self.device)
-        check(L.mtj_sample_nucleus(ptr(ses.logits), ses.B, self.w.V, ptr(top_p), ptr(temp), ptr(top_k), ptr(uniforms),
+        check(L.mtj_sample_nucleus(ptr(ses.logits if logits is None else logits), ses.B, self.w.V, ptr(top_p), ptr(temp), ptr(top_k), ptr(uniforms),
                                    uniforms.shape[1], ptr(ses.tok), ptr(out_tokens), out_tokens.shape[1], ptr(ses.pos),
                                    ptr(ses.pos_start), ptr(keep_mask), ptr(filtered), ptr(ses.sample_work),
                                    self._next(ses, embed_next), _abi.stream_handle()))

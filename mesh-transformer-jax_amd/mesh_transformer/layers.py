@@ -92,6 +92,35 @@ class EmbeddingShard:
             return torch.ops.mtj.embed(tok.reshape(-1).contiguous(), w, b)
 
 
+def _mask_geometry(attn_bias, t, T):
+    """What the kernels can apply of an additive attention bias [.., t, T]: the causal mask, plus `pad` masked leading
+    keys (the -1e10 terms that __call__, get_init_decode_state and decode_once build, layers.py:299-366).
+    Returns pad; anything else is not on this path."""
+    b = np.asarray(attn_bias.cpu() if isinstance(attn_bias, torch.Tensor) else attn_bias, dtype=np.float64)
+    if b.ndim == 0 or b.size == 1:
+        if float(b.reshape(-1)[0]) != 0.0:
+            raise NotImplementedError("a constant attention bias is not on the GPT-J path")
+        if t != 1:
+            raise NotImplementedError("attention without a causal mask (attn_bias = 0 on more than one query) has no kernel")
+        return 0
+    if b.shape[-1] != T or (b.ndim >= 2 and b.shape[-2] != t):
+        raise ValueError(f"attn_bias must broadcast to [heads, {t}, {T}]")
+    b = b.reshape(-1, t, T) if b.ndim >= 2 else np.broadcast_to(b, (1, t, T))
+    masked = b[0] < -1e9
+    if np.any(b != b[:1]) or np.any((b[0] != 0.0) & ~masked):
+        raise NotImplementedError("only masks of 0 / -1e10 shared by all heads are on the GPT-J path")
+    last = masked[-1]
+    pad = int(np.argmin(last)) if not last.all() else T
+    want = np.arange(T)[None, :] < pad
+    if t == T and T > 1:
+        want = want | (np.arange(T)[None, :] > np.arange(T)[:, None])
+    elif t != 1:
+        raise NotImplementedError("self_attn runs a whole window (t == T) or one new token (t == 1)")
+    if not np.array_equal(masked, np.broadcast_to(want, (t, T))):
+        raise NotImplementedError("attention bias is not causal + left padding")
+    return pad
+
+
 class TransformerLayerShard:
     """layers.py:229-366.  Returns the residual DELTA, like the reference; the caller adds x.
 
@@ -109,6 +138,84 @@ class TransformerLayerShard:
         self.eng = Engine(config, _tree(params), device, layer_ids=[self.index], embed=False, proj=False)
         self.dim, self.heads, self.dim_per_head = dim, heads, dim // heads
         self.pe_rotary_dims = config.get("pe_rotary_dims", self.dim_per_head)
+
+    # ---- the pieces of the layer (layers.py:260-297) on their own
+    def _h(self, x):
+        """float32 rows -> the GEMM operand type of this model (float16 saturates, as the kernels' own conversions do)"""
+        w = self.eng.w
+        x = _f32_in(x, self.eng.device).reshape(-1, w.d)
+        return x if w.act_torch_dtype == torch.float32 else x.clamp(-65504.0, 65504.0).to(w.act_torch_dtype)
+
+    def _scratch(self, T):
+        """Buffers of the piecewise entry points: a session of its own, so that the window of a live decode state (which
+        belongs to the engine's sessions) is never touched."""
+        from .engine import Session
+        ses = getattr(self, "_scratch_ses", None)
+        if ses is None or ses.Tcap != T:
+            self._scratch_ses = ses = None
+            ses = self._scratch_ses = Session(self.eng, 1, T, T, T + 1)
+        return ses
+
+    def qvk_proj(self, x):
+        """layers.py:292-297: q, v, k = x @ Wq, x @ Wv, x @ Wk (no bias) as [..., heads, d_head]; x is the LayerNorm output."""
+        eng, w = self.eng, self.eng.w
+        lead = tuple(np.shape(x)[:-1])
+        with torch.cuda.device(eng.device):
+            h = self._h(x)
+            out = torch.ops.mtj.gemm(h, w.w_in_mm[self.index][:3 * w.d], None, w.alpha_in[self.index], 0)  # rows q|v|k
+        d = w.d
+        return tuple(out[:, j * d:(j + 1) * d].reshape(lead + (self.heads, self.dim_per_head)) for j in range(3))
+
+    def self_attn(self, q, v, k, attn_bias):
+        """layers.py:260-285: rotary embedding of q and k at the window indices (q on the last rows), scores / sqrt(d_head)
+        + attn_bias, softmax, weighted values, output projection.  q [t, H, dh], v and k [T, H, dh] float32 and NOT yet
+        rotated; attn_bias must be what the layer drivers build: the causal mask (t == T) or none (t == 1), plus masked
+        leading keys.  Query rows that are themselves padding come back as the projection of zeros."""
+        eng, w, i = self.eng, self.eng.w, self.index
+        dev, H, dh, d = eng.device, self.heads, self.dim_per_head, w.d
+        q, v, k = (_f32_in(a, dev) for a in (q, v, k))
+        t, T = q.shape[0], k.shape[0]
+        pad = _mask_geometry(attn_bias, t, T)
+        A = w.act_dtype
+        with torch.cuda.device(dev):
+            ses = self._scratch(T)
+            kv_pos0 = torch.tensor([-pad], dtype=torch.int32, device=dev)
+            if t == T and T > 1:
+                torch.ops.mtj.rope_append_(q.reshape(T, d), v.reshape(T, d), k.reshape(T, d), kv_pos0, ses.sin, ses.cos,
+                                           ses.q_pf, ses.kc[i], ses.vc[i], ses.vt, H, self.pe_rotary_dims, T, ses.ldvt)
+                att = torch.ops.mtj.attn_prefill(ses.q_pf, ses.kc[i], ses.vt.view(1, H, dh, ses.ldvt), kv_pos0, T, None)
+            else:
+                q_pos = torch.tensor([T - 1 - pad], dtype=torch.int32, device=dev)
+                torch.ops.mtj.rope_append_(None, v.reshape(T, d), k.reshape(T, d), kv_pos0, ses.sin, ses.cos, None,
+                                           ses.kc[i], ses.vc[i], None, H, self.pe_rotary_dims, T, 0)
+                torch.ops.mtj.rope_append_(q.reshape(1, d), None, None, q_pos, ses.sin, ses.cos, ses.q, None, None, None,
+                                           H, self.pe_rotary_dims, 1, 0)
+                att = torch.ops.mtj.attn_decode(ses.q, ses.kc[i], ses.vc[i], q_pos, A)
+            # out projection: the out | fc_out matrix on [attention | 0]
+            act = ses.act_pf[:t]
+            act.zero_()
+            act[:, :d].copy_(att)
+            out = torch.zeros(t, d, dtype=torch.float32, device=dev)
+            torch.ops.mtj.gemm_resid_(out, act, w.w_out_mm[i], None, w.alpha_out[i])
+        return out
+
+    def ff(self, x):
+        """layers.py:287-290: gelu(x @ W1 + b1) @ W2 + b2 (tanh gelu); x is the LayerNorm output, [T, d]."""
+        eng, w, i = self.eng, self.eng.w, self.index
+        dev, d = eng.device, w.d
+        with torch.cuda.device(dev):
+            h = self._h(x)
+            T = h.shape[0]
+            ses = self._scratch(T)
+            act = ses.act_pf[:T]
+            pos0 = torch.zeros(1, dtype=torch.int32, device=dev)
+            # the fused q|v|k|fc_in launch: its fc_in columns are gelu(x @ W1 + b1); q, k, v land in the scratch window
+            torch.ops.mtj.inproj_(h, w.w_in_mm[i], w.b1[i], w.alpha_in[i], pos0, ses.sin, ses.cos, ses.q_pf, ses.kc[i],
+                                  ses.vc[i], None, act, self.heads, self.pe_rotary_dims, T, 0)
+            act[:, :d].zero_()
+            out = torch.zeros(T, d, dtype=torch.float32, device=dev)
+            torch.ops.mtj.gemm_resid_(out, act, w.w_out_mm[i], w.b2[i], w.alpha_out[i])
+        return out
 
     # ---- whole-layer entry points
     def _prefill(self, x, given_length):
@@ -170,3 +277,20 @@ class ProjectionShard:
         with torch.cuda.device(eng.device):
             h = torch.ops.mtj.layernorm(x, w.pln_s, w.pln_o, w.act_dtype)
             return torch.ops.mtj.gemm(h, w.w_p_mm, w.b_p, w.alpha_p, 0)
+
+    def loss(self, x, targets, z_loss=1):
+        """layers.py:569-593: per-row cross entropy of `targets` under the projected logits and `correct` (the target
+        holds the row maximum); with z_loss the mean over rows of 1e-4 * z_loss * log(sum exp(logits - max))^2 is added to
+        every row.  x float32 [T, d] (before the final LayerNorm), targets [T].  The [T, V] logits are never stored."""
+        eng, w = self.eng, self.eng.w
+        x = _f32_in(x, eng.device).reshape(-1, w.d)
+        tg = torch.as_tensor(np.asarray(targets).astype(np.int32) if not isinstance(targets, torch.Tensor) else targets)
+        tg = tg.to(eng.device, torch.int32).reshape(-1).contiguous()
+        with torch.cuda.device(eng.device):
+            h = torch.ops.mtj.layernorm(x, w.pln_s, w.pln_o, w.act_dtype)
+            loss, correct = torch.ops.mtj.gemm_xent(h, w.w_p_mm, w.b_p, w.alpha_p, tg)
+            if z_loss:
+                # a target outside the vocabulary selects nothing: the loss of such a row is its log-sum-exp
+                lse, _ = torch.ops.mtj.gemm_xent(h, w.w_p_mm, w.b_p, w.alpha_p, torch.full_like(tg, -1))
+                loss = loss + (1e-4 * float(z_loss)) * lse.square().mean()
+        return loss, correct

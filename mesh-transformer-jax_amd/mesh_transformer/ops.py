@@ -15,6 +15,7 @@ hop per launch would buy nothing).  Operators that write into caller-owned memor
     torch.ops.mtj.gemm_resid_(x, A, W, bias, alpha)                ... + residual add           layers.py:313
     torch.ops.mtj.gemv(x, W, bias, ln_scale, ln_offset)            hk.Linear on one row (+ LN)  layers.py:316-344
     torch.ops.mtj.inproj_(...)                                     fused q|v|k|fc_in projection layers.py:261-297,325-326
+    torch.ops.mtj.rope_append_(...)                                rotary + K/V window append   layers.py:261-273,325-326
     torch.ops.mtj.attn_prefill(q, k_cache, v_t, pos0, Tp, key_limit)   self_attn + masks        layers.py:260-285,347-366
     torch.ops.mtj.attn_decode(q, k_cache, v_cache, pos, out_dtype) one-token attention          layers.py:316-344
     torch.ops.mtj.xent(logits, target)                             ProjectionShard.loss         layers.py:569-593
@@ -152,6 +153,24 @@ def _inproj_(h, W, b1, alpha, pos0, sin_tab, cos_tab, q, k_cache, v_cache, v_t, 
                          _s()))
 
 
+def _rope_append_(q_in, v_in, k_in, pos0, sin_tab, cos_tab, q, k_cache, v_cache, v_t, n_heads, rotary_dims, Tp, ldvt):
+    """Rotary embedding + window append of projected rows (float32 [M, d] each, any may be None): what inproj_ does
+    after its GEMM.  Row m is token m % Tp of sequence m // Tp at position pos0[b] + t."""
+    src = next(t for t in (q_in, v_in, k_in) if t is not None)
+    M, d = src.shape
+    ip = InProj()
+    ip.n_heads, ip.d_head, ip.rotary_dims = n_heads, d // n_heads, rotary_dims
+    ref = k_cache if k_cache is not None else v_cache
+    ip.Tp, ip.Tcap, ip.max_pos = Tp, (ref.shape[2] if ref is not None else Tp), sin_tab.shape[0]
+    ip.pos0, ip.sin_tab, ip.cos_tab = ptr(pos0), ptr(sin_tab), ptr(cos_tab)
+    ip.q, ip.q_dtype = (ptr(q), _code(q)) if q is not None else (None, 0)
+    ip.kv_dtype = _code(ref) if ref is not None else 0
+    ip.k_cache, ip.v_cache = ptr(k_cache), ptr(v_cache)
+    ip.v_t, ip.ldvt = (ptr(v_t), ldvt) if v_t is not None else (None, 0)
+    srcs = [None if t is None else t.contiguous() for t in (q_in, v_in, k_in)]     # alive until the call is enqueued
+    check(_abi.lib().mtj_rope_append(ptr(srcs[0]), ptr(srcs[1]), ptr(srcs[2]), M, C.byref(ip), _s()))
+
+
 # ---------------------------------------------------------------- attention
 def _attn_prefill(q, k_cache, v_t, pos0, Tp, key_limit):
     B, H, Tcap, dh = k_cache.shape
@@ -177,7 +196,8 @@ def _sample_greedy(logits):
     R, V = logits.shape
     tok = torch.zeros(R, dtype=torch.int32, device=logits.device)
     pos = torch.zeros(R, dtype=torch.int32, device=logits.device)
-    check(_abi.lib().mtj_sample_greedy(ptr(logits), R, V, ptr(tok), None, 0, ptr(pos), ptr(pos.clone()), None, _s()))
+    pos_start = torch.zeros_like(pos)              # alive until the call has been enqueued
+    check(_abi.lib().mtj_sample_greedy(ptr(logits), R, V, ptr(tok), None, 0, ptr(pos), ptr(pos_start), None, _s()))
     return tok
 
 
@@ -189,12 +209,13 @@ def _sample_nucleus(logits, top_p, temp, top_k, uniforms):
     L = _abi.lib()
     tok = torch.zeros(R, dtype=torch.int32, device=dev)
     pos = torch.zeros(R, dtype=torch.int32, device=dev)
+    pos_start = torch.zeros_like(pos)
     filtered = torch.empty(R, V, dtype=torch.float32, device=dev)
     mask = torch.empty(R, V, dtype=torch.uint8, device=dev)
     work = torch.empty(L.mtj_sample_work_bytes(R, V), dtype=torch.uint8, device=dev)
     u = uniforms.reshape(R, 1).contiguous()
     check(L.mtj_sample_nucleus(ptr(logits), R, V, ptr(top_p), ptr(temp), ptr(top_k), ptr(u), 1, ptr(tok), None, 0, ptr(pos),
-                               ptr(pos.clone()), ptr(mask), ptr(filtered), ptr(work), None, _s()))
+                               ptr(pos_start), ptr(mask), ptr(filtered), ptr(work), None, _s()))
     return tok, filtered, mask.bool()
 
 
@@ -210,6 +231,9 @@ _define("gemv(Tensor x, Tensor W, Tensor? bias, Tensor? ln_scale, Tensor? ln_off
 _define("inproj_(Tensor h, Tensor W, Tensor b1, float alpha, Tensor pos0, Tensor sin_tab, Tensor cos_tab, Tensor(a!) q, "
         "Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor(d!)? v_t, Tensor(e!) act, int n_heads, int rotary_dims, int Tp, "
         "int ldvt) -> ()", _inproj_)
+_define("rope_append_(Tensor? q_in, Tensor? v_in, Tensor? k_in, Tensor pos0, Tensor sin_tab, Tensor cos_tab, Tensor(a!)? q, "
+        "Tensor(b!)? k_cache, Tensor(c!)? v_cache, Tensor(d!)? v_t, int n_heads, int rotary_dims, int Tp, int ldvt) -> ()",
+        _rope_append_)
 _define("attn_prefill(Tensor q, Tensor k_cache, Tensor v_t, Tensor pos0, int Tp, Tensor? key_limit) -> Tensor", _attn_prefill)
 _define("attn_decode(Tensor q, Tensor k_cache, Tensor v_cache, Tensor pos, int out_dtype) -> Tensor", _attn_decode)
 _define("sample_greedy(Tensor logits) -> Tensor", _sample_greedy)
@@ -217,4 +241,4 @@ _define("sample_nucleus(Tensor logits, Tensor top_p, Tensor temp, Tensor? top_k,
         _sample_nucleus)
 
 OPS = ("layernorm", "embed", "xent", "pack_weight", "pack_weight_f16", "gemm", "gemm_xent", "gemm_resid_", "gemv", "inproj_",
-       "attn_prefill", "attn_decode", "sample_greedy", "sample_nucleus")
+       "rope_append_", "attn_prefill", "attn_decode", "sample_greedy", "sample_nucleus")

@@ -89,7 +89,8 @@ def greedy_sample(key, logits, _, **unused):
     with torch.cuda.device(dev):
         tok = torch.zeros(R, dtype=torch.int32, device=dev)
         pos = torch.zeros(R, dtype=torch.int32, device=dev)
-        check(L.mtj_sample_greedy(ptr(lg), R, V, ptr(tok), None, 0, ptr(pos), ptr(pos.clone()), None, _abi.stream_handle()))
+        pos_start = torch.zeros_like(pos)
+        check(L.mtj_sample_greedy(ptr(lg), R, V, ptr(tok), None, 0, ptr(pos), ptr(pos_start), None, _abi.stream_handle()))
         torch.cuda.current_stream().synchronize()
     return (tok.cpu().numpy().astype(np.uint32) if is_np else tok), None
 
@@ -98,6 +99,8 @@ def builtin_kind(sampler):
     """Which fused device sampler a config["sampler"] callable maps to (None: call it on the host)."""
     if sampler is nucleaus_sample:
         return "nucleus"
+    if sampler is softmax_sample:
+        return "softmax"
     if sampler is greedy_sample:
         return "greedy"
     return None

@@ -55,6 +55,50 @@ def _to_device_tree(tree, device):
     return out
 
 
+class DecodeStates:
+    """The per-layer decode state that the reference's scan carries out of generate (transformer_shard.py:196-212,
+    layers.py:340-344): a sequence over the layers of {"k", "v": [B, T, H, dh], "tokens_decoded": uint32 [B]} with the
+    window in the reference's order (oldest slot first, the newest token last) and K NOT rotated.
+
+    The engine keeps K rotated at absolute positions in a ring, so an entry is computed (copied out of the ring,
+    rotated back) only when it is indexed; nothing is handed out that aliases the engine's memory.  Slots that still
+    hold left padding are zero (the reference keeps the projections of its pad tokens there, which no real token can
+    see).  Reading an entry after a later generate call on the same geometry raises: the window has moved on."""
+
+    def __init__(self, eng, ses, tokens_decoded):
+        self._eng, self._ses, self._epoch = eng, ses, ses.epoch
+        self._n = np.asarray(tokens_decoded).astype(np.int64)     # tokens in the window = next position, per sequence
+
+    def __len__(self):
+        return len(self._eng.w.layer_ids)
+
+    def __iter__(self):
+        return (self[i] for i in range(len(self)))
+
+    def __getitem__(self, layer):
+        eng, ses = self._eng, self._ses
+        if ses.epoch != self._epoch:
+            raise RuntimeError("this decode state belongs to an earlier generate call; the K/V window has been reused")
+        i = eng.w.layer_ids[layer]
+        T, dev, r = ses.Tcap, eng.device, eng.r
+        with torch.cuda.device(dev):
+            n = torch.from_numpy(self._n).to(dev)                                   # [B]
+            p = n[:, None] - T + torch.arange(T, device=dev)[None, :]               # position held by window slot j
+            real = p >= 0
+            slot = torch.where(real, p % T, torch.zeros_like(p))                    # [B, T]
+            idx = slot[:, None, :, None].expand(-1, eng.H, -1, eng.dh)
+            k = torch.gather(ses.kc[i], 2, idx).float()                             # [B, H, T, dh], rotated
+            v = torch.gather(ses.vc[i], 2, idx).float()
+            pp = p.clamp(0, ses.max_pos - 1)
+            sn, cs = ses.sin[pp][:, None], ses.cos[pp][:, None]                     # [B, 1, T, r/2]
+            ke, ko = k[..., 0:r:2].clone(), k[..., 1:r:2].clone()
+            k[..., 0:r:2] = ke * cs + ko * sn                                       # the rotation of layers.py:137-148, inverted
+            k[..., 1:r:2] = ko * cs - ke * sn
+            keep = real[:, None, :, None]
+            k, v = (k * keep).permute(0, 2, 1, 3), (v * keep).permute(0, 2, 1, 3)
+            return {"k": k.cpu().numpy(), "v": v.cpu().numpy(), "tokens_decoded": self._n.astype(np.uint32)}
+
+
 class CausalTransformer:
     """Drop-in for transformer_shard.py:118-339 on the generate path.
 
@@ -109,7 +153,9 @@ class CausalTransformer:
 
         ctx uint32 [B, L] left-padded (device_sample.py:92-96), ctx_length [B], sampler_options a dict of
         [B] arrays (top_p, temp, optional top_k).  Returns (final_state, (tokens [B, G, 1] uint32, None
-        [, logits [B, G, 1, V] float32])) so that callers' `out[1][0][:, :, 0]` works unchanged.
+        [, logits [B, G, 1, V] float32])) so that callers' `out[1][0][:, :, 0]` works unchanged.  final_state is the
+        scan's last carry (last token [B, 1], a sequence of per-layer {"k", "v", "tokens_decoded"}, None for the key);
+        the per-layer entries are built when they are read (see DecodeStates).
 
         Beyond the reference: `uniforms` float64 [B, G] in [0, 1) drive the inverse-CDF draw (default:
         drawn from an unseeded Philox stream, like the reference's unseeded key at :327);
@@ -149,12 +195,13 @@ class CausalTransformer:
             ses.tok.copy_(torch.from_numpy(ctx[:, -1].astype(np.int32)))
             ses.out_tokens.zero_()
             opts = dict(sampler_options or {})
-            if kind == "nucleus":
-                tp = np.broadcast_to(np.asarray(opts.get("top_p", 0.9), np.float64), (B,))
+            if kind in ("nucleus", "softmax"):
+                # softmax_sample (sampling.py:6-7) is the nucleus kernel with nothing filtered: top_p above 1, no top_k
+                tp = np.broadcast_to(np.asarray(opts.get("top_p", 0.9) if kind == "nucleus" else 2.0, np.float64), (B,))
                 tm = np.broadcast_to(np.asarray(opts.get("temp", 1.0), np.float64), (B,))
                 ses.top_p.copy_(torch.from_numpy(np.array(tp)))
                 ses.temp.copy_(torch.from_numpy(np.array(tm)))
-                tk = opts.get("top_k", None)
+                tk = opts.get("top_k", None) if kind == "nucleus" else None
                 ses.use_top_k = tk is not None
                 if ses.use_top_k:
                     ses.top_k.copy_(torch.from_numpy(np.array(np.broadcast_to(np.asarray(tk, np.int32), (B,)))))
@@ -195,11 +242,20 @@ class CausalTransformer:
                 timing.update(prefill_s=t1 - t0, prefill_tokens=B * Tp, warmup_s=t2 - t1, decode_s=t3 - t2,
                               decode_steps=G - W)
             torch.cuda.synchronize(dev)
-            if ses.oa_work is not None and int(ses.oa_work[8:12].view(torch.int32)[0]) != 0:
-                raise RuntimeError("a fused out-projection launch gave up waiting for its attention partials; "
-                                   "set config['fused_decode_attention'] = False")
+            if ses.fused_attn and int(ses.oa_work[8:12].view(torch.int32)[0]) != 0:
+                # a fused launch gave up its (time-bounded) wait: this call's tokens are void.  Clear the flag and
+                # keep this session on the separate attention launches from now on; the next call works.
+                ses.oa_work[8:12].zero_()
+                ses.fused_attn = False
+                ses.graphs = {}
+                torch.cuda.synchronize(dev)
+                raise RuntimeError("a fused out-projection launch gave up waiting for its attention partials (not all "
+                                   "of its workgroups were resident on the GPU within 5 ms); this call's output is "
+                                   "discarded and the session now uses separate attention launches - call generate again")
             toks = ses.out_tokens[:, :G].cpu().numpy().astype(np.uint32)[:, :, None]
-            final_state = (toks[:, -1], ses, None)
+            ses.epoch = getattr(ses, "epoch", 0) + 1
+            # the scan's final carry (transformer_shard.py:196-212): (last token, per-layer decode state, key)
+            final_state = (toks[:, -1], DecodeStates(eng, ses, P - 1 + G), None)
             out = (toks, None)
             if return_logits:
                 out = out + (logits_out.cpu().numpy()[:, :, None, :],)
@@ -287,18 +343,19 @@ class CausalTransformer:
             ses.use_top_k = False
             ses.graphs = {}
 
-    def _step(self, eng, ses, kind, keep_mask=None):
-        eng.decode_model(ses)
+    def _step(self, eng, ses, kind, keep_mask=None, logits=None):
+        eng.decode_model(ses, logits)
         if kind == "greedy":
-            eng.sample_greedy(ses, ses.out_tokens)
+            eng.sample_greedy(ses, ses.out_tokens, logits=logits)
         else:
             eng.sample_nucleus(ses, ses.out_tokens, ses.top_p, ses.temp, ses.top_k if ses.use_top_k else None,
-                               ses.uniforms, keep_mask=keep_mask)
+                               ses.uniforms, keep_mask=keep_mask, logits=logits)
 
     def _decode(self, eng, ses, t, G, kind, logits_out, masks):
-        """Decode steps t .. G-1."""
+        """Decode steps t .. G-1.  With logits_out the recorded steps write their logits into per-step slots of a
+        staging buffer (the same compiled program with one more output, like transformer_shard.py:205-208)."""
         spg = int(self.config.get("steps_per_graph", 8))
-        eager = spg <= 0 or logits_out is not None or masks is not None
+        eager = spg <= 0 or masks is not None
         while t < G:
             if eager or t == 0:
                 # the first step always runs eagerly: it also performs the kernels' one-time setup
@@ -308,21 +365,28 @@ class CausalTransformer:
                 t += 1
                 continue
             n = spg if G - t >= spg else 1
-            self._graph(eng, ses, kind, n).replay()
+            self._graph(eng, ses, kind, n, logits_out is not None).replay()
+            if logits_out is not None:
+                logits_out[:, t:t + n].copy_(ses.logits_stage[:n].transpose(0, 1))
             t += n
 
-    def _graph(self, eng, ses, kind, n):
-        key = (kind, n, ses.use_top_k)
+    def _graph(self, eng, ses, kind, n, with_logits=False):
+        key = (kind, n, ses.use_top_k, with_logits)
         g = ses.graphs.get(key)
         if g is None:
-            if kind == "nucleus" and ses.sample_work is None:
+            if kind != "greedy" and ses.sample_work is None:
                 ses.sample_work = torch.empty(_abi.lib().mtj_sample_work_bytes(ses.B, eng.w.V), dtype=torch.uint8,
                                               device=self.device)
+            if with_logits and (getattr(ses, "logits_stage", None) is None or ses.logits_stage.shape[0] < n):
+                for k in [k for k in ses.graphs if k[3]]:          # recorded against the buffer that is replaced
+                    del ses.graphs[k]
+                ses.logits_stage = torch.empty(max(n, int(self.config.get("steps_per_graph", 8))), ses.B, eng.w.V,
+                                               dtype=torch.float32, device=self.device)
             torch.cuda.synchronize(self.device)
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
-                for _ in range(n):
-                    self._step(eng, ses, kind)
+                for j in range(n):
+                    self._step(eng, ses, kind, logits=ses.logits_stage[j] if with_logits else None)
             ses.graphs[key] = g
         return g
 

@@ -345,10 +345,11 @@ class Model:
         return self.proj(x), new_states
 
     def generate(self, ctx, ctx_length, gen_length: int, sampler: Callable, sampler_options: dict,
-                 uniforms=None, return_logits=False):
+                 uniforms=None, return_logits=False, final_states: Optional[list] = None):
         """transformer_shard.py:190-216,326-339 - per sequence: prefill, then gen_length steps of
         generate_once + sampler.  sampler(u, logits[1,V] float32, **opts) -> uint32 token; `u` is the
-        step's host-supplied uniform (stands in for the reference's PRNG key)."""
+        step's host-supplied uniform (stands in for the reference's PRNG key).  final_states, a list, receives
+        the decode state each sequence ends with (the carry of transformer_shard.py:196-212)."""
         ctx = np.asarray(ctx)
         B = ctx.shape[0]
         toks = np.zeros((B, gen_length, 1), np.uint32)
@@ -365,6 +366,8 @@ class Model:
                 toks[b, t, 0] = tok
                 if return_logits:
                     logits_out[b, t] = lg32
+            if final_states is not None:      # the scan's last carry of this sequence: per-layer {k, v, tokens_decoded}
+                final_states.append(states)
         return (toks, None, logits_out) if return_logits else (toks, None)
 
 
@@ -435,6 +438,11 @@ def nucleaus_sample(u, logits, top_p=0.9, temp=1.0, top_k=None) -> int:
     """sampling.py:41-44 with the draw replaced: filter on raw logits, temperature after."""
     f = nucleaus_filter(logits, top_p, top_k)
     return inverse_cdf_draw(logits, f, temp, u)
+
+
+def softmax_sample(u, logits, temp=1.0) -> int:
+    """sampling.py:6-7 with the draw replaced: categorical over softmax(logits / temp), nothing filtered."""
+    return inverse_cdf_draw(logits, np.asarray(logits, np.float32), temp, u)
 
 
 def greedy_sample(u, logits, **_) -> int:

@@ -78,11 +78,14 @@ def test_full_context_forward_agrees_with_the_decode_path(net6b):
     assert float((l2[0, first:] - keep[-1:]).abs().max()) > 0.0
 
 
-def test_batch32_nucleus_decode_rows_are_independent(net6b):
-    """Batch 32, 1024-token prompts padded to 2048, top_p 0.9 / temperature 0.8, host Philox(3) uniforms: rows
-    with the same prompt and uniforms give the same stream wherever they sit in the batch, rows with different
-    uniforms do not, and every token id is a valid id."""
-    B, P, L, G = 32, 1024, 2048, 96
+def test_batch32_nucleus_decode_fills_the_window(net6b):
+    """BASELINE config 4 at its real length: batch 32, 1024-token prompts padded to 2048, 1024 generated tokens (the
+    K/V window fills to 2047 keys, layers.py:316-344), top_p 0.9 / temperature 0.8, host Philox(3) uniforms.  Rows
+    with the same prompt and uniforms give the same stream wherever they sit in the batch, over all 1024 steps; rows
+    with different uniforms do not; every token id is valid; and the logits of the FIRST and of the LAST step agree
+    within 2e-2 with a batch-2 run of the same rows (the last step teacher-forced: the rows' prompt followed by what
+    they generated, through the prefill kernels instead of 1023 decode steps)."""
+    B, P, L, G = 32, 1024, 2048, 1024
     u = np.random.Generator(np.random.Philox(3)).random((B, G))
     ids = np.random.Generator(np.random.Philox(33)).integers(0, 50257, (B, P))
     ids[17] = ids[0]
@@ -91,11 +94,14 @@ def test_batch32_nucleus_decode_rows_are_independent(net6b):
     ctx = np.zeros((B, L), np.uint32)
     ctx[:, L - P:] = ids
     opts = {"top_p": np.full(B, 0.9), "temp": np.full(B, 0.8)}
-    tm = {"warmup": 9}
-    _, out = net6b.generate(ctx, np.full(B, P), G, opts, uniforms=u, timing=tm, return_logits=True)
+    tm = {"warmup": G - 64}
+    _, out = net6b.generate(ctx, np.full(B, P), G, opts, uniforms=u, timing=tm)
     toks = out[0][:, :, 0]
-    print(f"batch-32 nucleus decode: {tm['decode_s'] / tm['decode_steps'] * 1e3:.3f} ms/step, "
-          f"{B * tm['decode_steps'] / tm['decode_s']:.0f} tok/s")
+    ses = net6b.engine().sessions[(B, L - 1)]
+    last_logits = ses.logits[[0, 4]].cpu().numpy()              # what the last step sampled from
+    assert int(ses.pos[0]) == P - 1 + G                         # 2047 positions written: the window is full
+    print(f"batch-32 nucleus decode, 1024 steps: {(tm['warmup_s'] + tm['decode_s']) / G * 1e3:.3f} ms/step overall, "
+          f"{tm['decode_s'] / tm['decode_steps'] * 1e3:.3f} ms/step over the last {tm['decode_steps']} (about 2015 keys)")
     assert toks.shape == (B, G) and toks.max() < 50400
     assert np.array_equal(toks[0], toks[17])
     assert not np.array_equal(toks[4], toks[9])           # same prompt, different uniforms
@@ -103,10 +109,20 @@ def test_batch32_nucleus_decode_rows_are_independent(net6b):
     # the logits of the first step, whose inputs are the prompt alone, agree within 2e-2.  (The sampled
     # streams need not: with a flat random-init distribution the nucleus holds thousands of tokens and a logit
     # change of 1e-3 moves the inverse-CDF draw to a neighbour.)
-    _, out2 = net6b.generate(ctx[[0, 4]], [P, P], 2, {"top_p": np.full(2, 0.9), "temp": np.full(2, 0.8)},
-                             uniforms=u[[0, 4], :2], return_logits=True)
-    d = np.abs(out2[2][:, 0, 0] - out[2][[0, 4], 0, 0]).max()
+    o2 = {"top_p": np.full(2, 0.9), "temp": np.full(2, 0.8)}
+    first = net6b.generate(ctx[[0, 4]], [P, P], 1, o2, uniforms=u[[0, 4], :1], return_logits=True)[1][2][:, 0, 0]
+    ref_first = net6b.generate(ctx, np.full(B, P), 1, opts, uniforms=u[:, :1], return_logits=True)[1][2][[0, 4], 0, 0]
+    d = np.abs(first - ref_first).max()
     print("first-step logits, batch 2 against batch 32: max |d|", d)
+    assert d < 2e-2
+    # last step: rows 0 and 4 again, their prompt followed by the 1023 tokens they generated, one decode step
+    ctx_l = np.zeros((2, L), np.uint32)
+    for j, b in enumerate((0, 4)):
+        ctx_l[j, 1:1 + P] = ids[b]
+        ctx_l[j, 1 + P:] = toks[b, :G - 1]
+    lastb2 = net6b.generate(ctx_l, [L - 1, L - 1], 1, o2, uniforms=u[[0, 4], :1], return_logits=True)[1][2][:, 0, 0]
+    d = np.abs(lastb2 - last_logits).max()
+    print("last-step logits (2047 keys), batch-2 teacher-forced prefill against 1023 batch-32 decode steps: max |d|", d)
     assert d < 2e-2
 
 

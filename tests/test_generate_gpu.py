@@ -348,3 +348,156 @@ def test_generate_argument_checks():
     with pytest.raises(ValueError):
         from mesh_transformer.transformer_shard import CausalTransformer
         CausalTransformer(dict(cfg, cores_per_replica=8))
+
+
+def test_fused_decode_attention_give_up_is_raised_once_and_recovered_from():
+    """The batch-1 out projection that computes the attention itself waits for its partials for a bounded time and
+    flags a give-up in word 2 of its counter block.  The flag is forced from the host here (every kernel still exits
+    normally: a launch that finds the flag up does not wait): generate must raise once, clear the flag, move the
+    session to the separate attention launches, and the next call must match the oracle again."""
+    from mesh_transformer import sampling
+    cfg = dict(layers=2, d_model=2048, n_heads=32, n_vocab=2048, norm="layernorm", pe="rotary", pe_rotary_dims=32,
+               seq=64, cores_per_replica=1)            # float32, K = 5 whole tiles: the fused kernel applies
+    params = O.seeded_params(cfg, 21)
+    ctx = O.left_pad(O.seeded_prompt(21, 1, 20, hi=2048), 64)
+    net = net_for(cfg, params, sampling.greedy_sample)
+    ref = O.Model(cfg, params, torch.float64).generate(ctx, [20], 12, O.greedy_sample, {})
+    _, out = net.generate(ctx, [20], 12, {})
+    ses = net.engine().sessions[(1, 63)]
+    assert ses.fused_attn and np.array_equal(out[0], ref[0])
+    flag = ses.oa_work[8:12].view(torch.int32)
+    assert int(flag[0]) == 0
+    flag.fill_(1)
+    with pytest.raises(RuntimeError, match="gave up"):
+        net.generate(ctx, [20], 12, {})
+    assert int(flag[0]) == 0 and not ses.fused_attn and not ses.graphs
+    _, again = net.generate(ctx, [20], 12, {})
+    assert net.engine().sessions[(1, 63)] is ses and np.array_equal(again[0], ref[0])
+
+
+@pytest.mark.parametrize("which", ["fp32", "bf16"])
+def test_layer_pieces_qvk_proj_self_attn_ff_and_projection_loss(which):
+    """The module-level seams of layers.py:260-297 and 569-593 one by one against the float64 oracle: qvk_proj,
+    self_attn on a whole left-padded window (causal + pad bias, as get_init_decode_state builds it) and on one new
+    token (pad bias only, as decode_once builds it), ff, and ProjectionShard.loss with and without z_loss - the loss
+    reference is the library cross entropy plus the z term written out on the oracle's logits."""
+    from mesh_transformer import layers
+    from mesh_transformer.layers import TransformerLayerShard, ProjectionShard
+    cfg, dt, tol = (CFG1, torch.float32, 1e-4) if which == "fp32" else (CFG_BF, torch.bfloat16, 4e-3)
+    params = O.seeded_params(cfg, 31, dt)
+    model = O.Model(cfg, params, torch.float64)
+    lref = model.layers[1]
+    g = torch.Generator().manual_seed(31)
+    T, pad = 45, 7
+    x = torch.randn(T, cfg["d_model"], generator=g, dtype=torch.float64)
+    xn = lref.norm(x)
+    with layers.transform(params):
+        layer = TransformerLayerShard(cfg, "layer_1", 2.0 / cfg["layers"])
+        proj = ProjectionShard(cfg)
+    q, v, k = layer.qvk_proj(xn.float())
+    qr, vr, kr = lref.qvk_proj(xn)
+    H, dh = cfg["n_heads"], cfg["d_model"] // cfg["n_heads"]
+    assert tuple(q.shape) == (T, H, dh)
+    for got, ref in ((q, qr), (v, vr), (k, kr)):
+        assert rel(got, ref) < tol
+    # whole window: causal mask + masked leading keys
+    bias = O.MASK * (1.0 - torch.tril(torch.ones(T, T, dtype=torch.float64)))
+    bias = bias - 1e10 * (torch.arange(T) < pad).double()
+    a_ref = lref.self_attn(qr, vr, kr, bias)
+    a_got = layer.self_attn(qr.float(), vr.float(), kr.float(), bias.numpy())
+    assert rel(a_got[pad:], a_ref[pad:]) < tol
+    # one new token against the window (decode_once): q is the last row, rotated at the last window index
+    bias1 = -1e10 * (torch.arange(T) < pad).double()
+    d_ref = lref.self_attn(qr[-1:], vr, kr, bias1)
+    d_got = layer.self_attn(qr[-1:].float(), vr.float(), kr.float(), bias1.numpy())
+    assert rel(d_got, d_ref) < tol
+    assert rel(d_got, a_ref[-1:]) < tol                       # the same thing, computed by the other kernel
+    with pytest.raises(NotImplementedError):
+        layer.self_attn(qr.float(), vr.float(), kr.float(), 0)                # several queries without a causal mask
+    with pytest.raises(NotImplementedError):
+        layer.self_attn(qr.float(), vr.float(), kr.float(), (bias * 1e-12).numpy())   # not a 0 / -1e10 mask
+    assert rel(layer.ff(xn.float()), lref.ff(xn)) < tol
+    # ProjectionShard.loss
+    tgt = torch.randint(0, cfg["n_vocab"], (T,), generator=g)
+    logits = model.proj(x)
+    tgt[3] = int(logits[3].argmax())                          # one row whose target holds the maximum
+    ce = torch.nn.functional.cross_entropy(logits, tgt, reduction="none")
+    lse = torch.logsumexp(logits - logits.max(-1, keepdim=True).values, -1)
+    for z in (0.0, 1.0, 2.5):
+        loss, correct = proj.loss(x.float(), tgt.numpy(), z)
+        ref = ce + (1e-4 * lse ** 2 * z).mean()
+        assert float((loss.double().cpu() - ref).abs().max()) < (1e-4 if which == "fp32" else 2e-2) * float(ref.abs().max())
+        assert bool(correct[3]) and np.array_equal(correct.cpu().numpy(), (logits.argmax(-1) == tgt).numpy())
+
+
+def test_softmax_sample_is_a_device_sampler():
+    """config["sampler"] = softmax_sample (sampling.py:6-7) runs on the fused device sampler (nothing filtered) and
+    follows the oracle's stream on the same uniforms; per-row temperatures."""
+    from mesh_transformer import sampling
+    assert sampling.builtin_kind(sampling.softmax_sample) == "softmax"
+    cfg = dict(CFG1, n_vocab=2048)
+    params = O.seeded_params(cfg, 14)
+    ctx = O.left_pad(O.seeded_prompt(14, 2, 21, hi=2048), 40)
+    G = 10
+    u = np.random.Generator(np.random.Philox(14)).random((2, G))
+    opts = {"temp": np.array([0.7, 1.4])}
+    net = net_for(cfg, params, sampling.softmax_sample)
+    _, out = net.generate(ctx, [21, 21], G, opts, uniforms=u)
+    ref = O.Model(cfg, params, torch.float64).generate(ctx, [21, 21], G, O.softmax_sample, opts, uniforms=u)
+    assert np.array_equal(out[0], ref[0])
+    assert len({int(t) for t in out[0].reshape(-1)}) > 4       # a draw, not an argmax
+
+
+@pytest.mark.parametrize("case", ["padded", "sliding"])
+def test_generate_returns_the_scan_carry(case):
+    """The first return value of generate (transformer_shard.py:196-216): last token, per-layer decode state in the
+    reference's layout ([B, T, H, dh], window order, K not rotated, tokens_decoded), key."""
+    from mesh_transformer import sampling
+    cfg = dict(CFG1, n_vocab=1024)
+    params = O.seeded_params(cfg, 15)
+    if case == "padded":
+        lens, L, G = [9, 14], 32, 6
+    else:
+        lens, L, G = [12, 12], 12, 5                            # the window slides: the oldest tokens are evicted
+    ctx = np.zeros((2, L), np.uint32)
+    for b, n in enumerate(lens):
+        ctx[b, L - n:] = O.seeded_prompt(50 + b, 1, n, hi=1024)[0]
+    net = net_for(cfg, params, sampling.greedy_sample)
+    final, out = net.generate(ctx, lens, G, {})
+    ref_states = []
+    ref = O.Model(cfg, params, torch.float64).generate(ctx, lens, G, O.greedy_sample, {}, final_states=ref_states)
+    assert np.array_equal(out[0], ref[0])
+    last, states, key = final
+    assert key is None and last.shape == (2, 1) and np.array_equal(last, ref[0][:, -1])
+    assert len(states) == cfg["layers"]
+    T = L - 1
+    for i, st in enumerate(states):
+        assert st["k"].shape == (2, T, cfg["n_heads"], 64) and st["tokens_decoded"].dtype == np.uint32
+        for b, n in enumerate(lens):
+            r = ref_states[b][i]
+            assert int(st["tokens_decoded"][b]) == r["tokens_decoded"] == n - 1 + G
+            real = min(n - 1 + G, T)
+            assert rel(st["k"][b, T - real:], r["k"][T - real:]) < 1e-5
+            assert rel(st["v"][b, T - real:], r["v"][T - real:]) < 1e-5
+            assert not st["k"][b, :T - real].any()
+    net.generate(ctx, lens, G, {})
+    with pytest.raises(RuntimeError):
+        states[0]                                               # the window has been reused by the later call
+
+
+def test_logits_from_the_graph_path_equal_the_eager_ones():
+    """return_logits keeps the recorded steps (the logits of a step go to a slot of a staging buffer); the eager
+    path (steps_per_graph = 0) must give the same bits, replay after replay."""
+    from mesh_transformer import sampling
+    cfg = dict(CFG1, n_vocab=4096)
+    params = O.seeded_params(cfg, 16)
+    ctx = O.left_pad(O.seeded_prompt(16, 2, 19, hi=4096), 64)
+    u = np.random.Generator(np.random.Philox(16)).random((2, 27))
+    opts = {"top_p": np.array([0.9, 0.8]), "temp": np.array([0.8, 1.1])}
+    eager = net_for(dict(cfg, steps_per_graph=0), params, sampling.nucleaus_sample)
+    _, ref = eager.generate(ctx, [19, 19], 27, opts, return_logits=True, uniforms=u)
+    net = net_for(cfg, params, sampling.nucleaus_sample)
+    for _ in range(2):
+        _, out = net.generate(ctx, [19, 19], 27, opts, return_logits=True, uniforms=u)
+        assert np.array_equal(out[0], ref[0]) and np.array_equal(out[2], ref[2])
+    assert any(k[3] for k in net.engine().sessions[(2, 63)].graphs)

@@ -294,6 +294,17 @@ def test_inverse_cdf_draw_brute_force_and_chi_square():
     assert chi2 < 30, chi2       # dof <= 6; P(chi2 > 30) ~ 4e-5
 
 
+def test_softmax_sample_follows_the_library_softmax():
+    """softmax_sample (sampling.py:6-7): the empirical distribution of the draw is torch.softmax(logits / temp)."""
+    rng = np.random.default_rng(5)
+    l = rng.standard_normal((1, 6)).astype(np.float32) * 1.5
+    temp, n = 1.3, 40000
+    p = torch.softmax(torch.from_numpy(l[0]).double() / temp, -1).numpy()
+    counts = np.bincount([O.softmax_sample(u, l, temp=temp) for u in rng.random(n)], minlength=6)
+    chi2 = ((counts - n * p) ** 2 / (n * p)).sum()
+    assert chi2 < 28, chi2       # dof 5; P(chi2 > 28) ~ 4e-5
+
+
 def test_greedy_lowest_index_on_ties():
     assert O.greedy_sample(None, np.array([[1.0, 3.0, 3.0, 2.0]], np.float32)) == 1
 

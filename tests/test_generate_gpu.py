@@ -501,3 +501,94 @@ def test_logits_from_the_graph_path_equal_the_eager_ones():
         _, out = net.generate(ctx, [19, 19], 27, opts, return_logits=True, uniforms=u)
         assert np.array_equal(out[0], ref[0]) and np.array_equal(out[2], ref[2])
     assert any(k[3] for k in net.engine().sessions[(2, 63)].graphs)
+
+
+# ------------------------------------------------------------------ float16 range: outlier channels, large LayerNorm scales
+def outlier_params(cfg, seed, saturate=False):
+    """A bf16 tree shaped like a trained model rather than like an initialiser: four residual channels carry +-50 ..
+    +-500 from the embedding bias on and grow by the fc_out bias in every layer (past 1000 at the end), LayerNorm scales
+    run from 0.5 to 30 with offsets ~N(0, 0.5), the input matrices are rescaled so that LayerNorm outputs reach ~40,
+    q and k ~25, attention scores a standard deviation of 1-11, fc_in ~50, the embedding matrix has entries up to ~5
+    and one k matrix holds +-4 next to N(0, 0.02) entries (its float16 copy gets a small power-of-two scale).
+    saturate: one fc_in bias of 1e5, so that one gelu output lies beyond the float16 range."""
+    p = O.seeded_params(cfg, seed, torch.float32)
+    rng = np.random.Generator(np.random.Philox(seed + 1000))
+    d = cfg["d_model"]
+    ch = np.array([7, 300, 511, 900])
+    big = np.array([300.0, -500.0, 50.0, -120.0], np.float32)
+    p[O.EMBED]["w"][0] *= 50.0
+    p[O.EMBED]["b"][0, ch] = torch.from_numpy(big)
+    for i in range(cfg["layers"]):
+        ln = p[O.layer_key(i, "replicated_layer_norm")]
+        sc = rng.uniform(0.5, 30.0, d).astype(np.float32)
+        sc[ch] = 1.0
+        ln["scale"][0] = torch.from_numpy(sc)
+        ln["offset"][0] = torch.from_numpy(rng.standard_normal(d).astype(np.float32) * 0.5)
+        p[O.layer_key(i, "linear_5")]["b"][0, ch] += torch.from_numpy(big * 0.3)
+        for name, gain in (("linear", 2.0), ("linear_1", 8.0), ("linear_2", 2.0), ("linear_4", 10.0)):
+            p[O.layer_key(i, name)]["w"][0] *= gain / torch.from_numpy(np.sqrt(sc))[:, None]
+    w = p[O.layer_key(1, "linear_2")]["w"]
+    w[0, 5, 17], w[0, 700, 333] = 4.0, -4.0
+    p[O.PROJ_LN]["scale"][0] = torch.from_numpy(rng.uniform(0.5, 3.0, d).astype(np.float32))
+    p[O.PROJ_LN]["offset"][0] = torch.from_numpy(rng.standard_normal(d).astype(np.float32) * 0.2)
+    if saturate:
+        p[O.layer_key(0, "linear_4")]["b"][0, 5] = 1.0e5
+    return {m: {k: v.to(torch.bfloat16) for k, v in l.items()} for m, l in p.items()}
+
+
+def test_outlier_channels_and_large_layernorm_scales_stay_within_the_bf16_bound():
+    """The matrix-core paths round their operands to float16 (5 exponent bits).  With the outlier tree above every
+    path must still be within 2e-2 of the float64 oracle on the logits: batch-1 generate (float32 activations at
+    decode, float16 in its prefill), batch-2 generate (float16 everywhere), the every-position forward, and eval."""
+    from mesh_transformer import sampling
+    params = outlier_params(CFG_BF, 77)
+    m = O.Model(CFG_BF, params, torch.float64)
+    net = net_for(CFG_BF, params, sampling.greedy_sample)
+    prompt = O.seeded_prompt(77, 2, 64)
+    ctx = O.left_pad(prompt, 128)
+    ctx[1, :64 + 23] = 0                                        # row 1 keeps 41 tokens
+    lens = [64, 41]
+    G = 12
+    for rows in ([0], [0, 1]):
+        c, n = ctx[rows], [lens[r] for r in rows]
+        _, out = net.generate(c, n, G, {}, return_logits=True)
+        ref_t, _, ref_l = m.generate(c, n, G, O.greedy_sample, {}, return_logits=True)
+        # teacher forcing is not needed while the streams agree; compare up to the first difference (if any)
+        same = (out[0] == ref_t).all(axis=(0, 2))
+        upto = G if same.all() else int(np.argmin(same)) + 1
+        err = float(np.abs(out[2][:, :upto] - ref_l[:, :upto]).max())
+        print(f"outliers, batch {len(rows)}: max |dlogit| {err:.2e} over {upto} steps; logits std {ref_l.std():.2f} max {np.abs(ref_l).max():.1f}")
+        assert err < 2e-2 and upto >= 8
+    toks = O.seeded_prompt(78, 1, 96)
+    got = net.forward(toks)[0].double().cpu()
+    ref = m.forward(toks[0])
+    err = float((got - ref).abs().max())
+    print(f"outliers, forward: max |dlogit| {err:.2e}; residual stream reaches {float(m.embed(toks[0]).abs().max()):.0f} at the input")
+    assert err < 2e-2
+    tgt = np.roll(toks, -1, axis=1)
+    ev = net.eval({"obs": toks, "target": tgt})
+    rl = m.loss(toks[0], tgt[0])
+    assert float(np.abs(ev["all_loss"][0] - rl["all_loss"].numpy()).max()) < 2e-2
+
+
+def test_operands_beyond_the_float16_range_saturate_and_stay_finite():
+    """One gelu output of 1e5 (an fc_in bias of 1e5): on the matrix-core paths that operand is 65504 - conversions to
+    float16 saturate instead of overflowing to infinity - so the caller sees finite logits, equal (within the usual
+    2e-2) to the reference evaluated with that operand clamped to +-65504, and not to the unclamped reference.  The
+    batch-1 decode step keeps float32 activations and does not clamp."""
+    from mesh_transformer import sampling
+    params = outlier_params(CFG_BF, 79, saturate=True)
+    net = net_for(CFG_BF, params, sampling.greedy_sample)
+    toks = O.seeded_prompt(79, 1, 48)
+    got = net.forward(toks)[0].double().cpu()
+    assert bool(torch.isfinite(got).all())
+    m = O.Model(CFG_BF, params, torch.float64)
+    free = m.forward(toks[0])
+    l0 = m.layers[0]
+    l0.ff = lambda x: torch.clamp(O.gelu_tanh(x @ l0.w1 + l0.b1), -65504.0, 65504.0) @ l0.w2 + l0.b2
+    clamped = m.forward(toks[0])
+    e_c, e_f = float((got - clamped).abs().max()), float((got - free).abs().max())
+    print(f"saturating operand: max |dlogit| vs clamped reference {e_c:.2e}, vs unclamped {e_f:.2e}")
+    assert e_c < 2e-2 < e_f
+    _, out = net.generate(O.left_pad(toks, 64), [48], 4, {}, return_logits=True)
+    assert np.isfinite(out[2]).all()

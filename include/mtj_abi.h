@@ -243,7 +243,10 @@ int mtj_attn_decode_partials(const float* q, const void* k_cache, const void* v_
  * live in a device array built into the library (MTJ_ATTN_DECODE_STATIC_BYTES per device, held until the process
  * ends: room for 4032 (sequence, head) pairs at d_head 256, e.g. batch 252 of a 16-head model); the call allocates nothing and returns MTJ_ELIMIT when mtj_attn_decode_work_bytes(B, H, dh, Tcap) exceeds
  * that.  Same arguments and results as mtj_attn_decode otherwise.  Every call on a device shares the array: calls
- * that overlap on one device (two streams, two threads) race. */
+ * that overlap on one device (two streams, two threads) race; nothing checks for it.
+ * Before the first capture on a device, call mtj_attn_decode_static_max_bytes() (or the entry point itself, eagerly,
+ * once per shape) with that device current: the array's address is looked up at the first use on a device and the
+ * kernels' attributes are set at their first launch, neither of which belongs inside a stream capture. */
 #define MTJ_ATTN_DECODE_STATIC_BYTES (4 * 1024 * 1024)
 int64_t mtj_attn_decode_static_max_bytes(void);
 int mtj_attn_decode_static(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos, int64_t B,

@@ -31,6 +31,20 @@ template <> struct mma<bf16_t> {
   __device__ static __forceinline__ floatx16 first(const frag& a, const frag& b) {   // product alone: C is the constant 0
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, floatx16{}, 0, 0, 0);
   }
+  // The same instruction spelled out, with the accumulator tied to vector registers (_v) or held in accumulation
+  // registers that are named here and nowhere else (_fixed), for a kernel that fills the whole register file and cannot
+  // leave the placement of its accumulators (and the copies it can entail) to the compiler.  The compiler does not know these are matrix instructions: the caller inserts the
+  // wait states before other instructions read the result.
+  __device__ static __forceinline__ void first_v(floatx16& c, const frag& a, const frag& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a.v), "v"(b.v));   // the result must not overlap an operand
+  }
+  __device__ static __forceinline__ void run_v(floatx16& c, const frag& a, const frag& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a.v), "v"(b.v));
+  }
+  // accumulator in the sixteen accumulation registers from a[BASE] on, which the compiler never sees
+  template <int BASE> __device__ static __forceinline__ void run_fixed(const frag& a, const frag& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 a[%c2:%c2+15], %0, %1, a[%c2:%c2+15]" : : "v"(a.v), "v"(b.v), "n"(BASE));
+  }
 };
 template <> struct mma<f16_t> {
   static constexpr int EPC = 8;
@@ -54,6 +68,20 @@ template <> struct mma<f16_t> {
   }
   __device__ static __forceinline__ floatx16 first(const frag& a, const frag& b) {   // product alone: C is the constant 0
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a.v, b.v, floatx16{}, 0, 0, 0);
+  }
+  // The same instruction spelled out, with the accumulator tied to vector registers (_v) or held in accumulation
+  // registers that are named here and nowhere else (_fixed), for a kernel that fills the whole register file and cannot
+  // leave the placement of its accumulators (and the copies it can entail) to the compiler.  The compiler does not know these are matrix instructions: the caller inserts the
+  // wait states before other instructions read the result.
+  __device__ static __forceinline__ void first_v(floatx16& c, const frag& a, const frag& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a.v), "v"(b.v));   // the result must not overlap an operand
+  }
+  __device__ static __forceinline__ void run_v(floatx16& c, const frag& a, const frag& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a.v), "v"(b.v));
+  }
+  // accumulator in the sixteen accumulation registers from a[BASE] on, which the compiler never sees
+  template <int BASE> __device__ static __forceinline__ void run_fixed(const frag& a, const frag& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 a[%c2:%c2+15], %0, %1, a[%c2:%c2+15]" : : "v"(a.v), "v"(b.v), "n"(BASE));
   }
 };
 template <> struct mma<float> {
@@ -677,6 +705,377 @@ __global__ __launch_bounds__(512) void attn_prefill_pair_kernel(const T* __restr
 }
 
 // ------------------------------------------------------------------------------------------------
+// Prefill for 16-bit types at d_head 256, long prompts: ONE wavefront per SIMD that owns 64 queries (two blocks of 32)
+// and does everything for them, four wavefronts = 256 queries per workgroup.  With 32 queries per wavefront (the pair
+// kernel above) every 1 KiB K or V^T fragment read from LDS feeds one matrix instruction, and LDS traffic (~200 KB per
+// 32-key tile and CU for 1024 matrix-pipe cycles) is what bounds that kernel; here a fragment feeds two, one per query
+// block, for the price of the register budget of a whole SIMD: Q 128 registers, the output accumulator 256, scores 32,
+// probabilities of two tiles 32.  The matrix pipe and the vector unit overlap inside the wavefront instead of across
+// a pair: iteration i first computes the scores of tile i (K Q^T), then issues the products V^T P^T of tile i-1
+// together with the softmax arithmetic of tile i, which the matrix instructions (32 cycles apiece, asynchronous) hide.
+// Same lane layout, K row permutation, LDS stages, xor swizzles and global -> LDS loads as the pair kernel; one
+// workgroup barrier per tile.
+constexpr int Q64_LDS_BYTES = PP_STAGES * (PP_KTILE + PP_VTILE);
+
+// The output accumulator of attn_prefill_q64_kernel lives in all 256 accumulation registers, addressed by number from
+// inline assembly only: block (qb, n) - 32 head dims x 32 queries - is a[(qb * 8 + n) * 16 .. + 15].  The clobber list
+// names every one of them once, which takes them out of the compiler's hands for good (it uses accumulation registers
+// that the function does not mention as spill space for vector registers).
+#define Q64_A8(n) "a" #n "0", "a" #n "1", "a" #n "2", "a" #n "3", "a" #n "4", "a" #n "5", "a" #n "6", "a" #n "7", "a" #n "8", "a" #n "9"
+#define Q64_ALL_ACC                                                                                                      \
+  "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", Q64_A8(1), Q64_A8(2), Q64_A8(3), Q64_A8(4), Q64_A8(5),     \
+      Q64_A8(6), Q64_A8(7), Q64_A8(8), Q64_A8(9), Q64_A8(10), Q64_A8(11), Q64_A8(12), Q64_A8(13), Q64_A8(14), Q64_A8(15), \
+      Q64_A8(16), Q64_A8(17), Q64_A8(18), Q64_A8(19), Q64_A8(20), Q64_A8(21), Q64_A8(22), Q64_A8(23), Q64_A8(24),         \
+      "a250", "a251", "a252", "a253", "a254", "a255"
+__device__ __forceinline__ void acc_zero_all() {
+  asm volatile(".set mtj_r, 0\n\t.rept 256\n\tv_accvgpr_write_b32 a[mtj_r], 0\n\t.set mtj_r, mtj_r+1\n\t.endr" : : : Q64_ALL_ACC);
+}
+template <int BASE> __device__ __forceinline__ void acc_scale16(float f) {        // a[BASE .. BASE+15] *= f
+  float tmp;
+  asm volatile(".set mtj_r, %c2\n\t.rept 16\n\tv_accvgpr_read_b32 %0, a[mtj_r]\n\tv_mul_f32 %0, %0, %1\n\t"
+               "v_accvgpr_write_b32 a[mtj_r], %0\n\t.set mtj_r, mtj_r+1\n\t.endr"
+               : "=&v"(tmp) : "v"(f), "n"(BASE));
+}
+template <int R> __device__ __forceinline__ float acc_read() {
+  float t;
+  asm volatile("v_accvgpr_read_b32 %0, a[%c1]" : "=v"(t) : "n"(R));
+  return t;
+}
+// max(a, b, c) in one instruction; the operands come out of matrix instructions, where the compiler would first
+// canonicalise each of them
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+// two probabilities -> one word of 16-bit operands, no clamp: they are at most 64 wherever the result is used
+template <typename T> __device__ __forceinline__ uint32_t pack_prob(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack_prob<bf16_t>(float lo, float hi) { return pack_bf16x2(lo, hi); }
+template <> __device__ __forceinline__ uint32_t pack_prob<f16_t>(float lo, float hi) {
+  const f16x2 r = {(f16_t)lo, (f16_t)hi};
+  return __builtin_bit_cast(uint32_t, r);
+}
+// f(integral_constant<int, K>) for K = 0 .. N-1, in order
+template <int N, int K = 0, class F> __device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (K < N) {
+    f(std::integral_constant<int, K>{});
+    static_for<N, K + 1>(f);
+  }
+}
+
+
+template <typename T>
+__global__ __launch_bounds__(256) void attn_prefill_q64_kernel(const T* __restrict__ q, const T* __restrict__ kc,
+                                                               const T* __restrict__ vt, const int32_t* __restrict__ pos0,
+                                                               int H, int Tp, int Tcap, int64_t ldvt, T* __restrict__ out,
+                                                               int64_t ld_out, int nseq, int nqblk,
+                                                               const int32_t* __restrict__ key_limit) {
+  static_assert(sizeof(T) == 2, "16-bit types");
+  constexpr int DH = 256, BKV = 32, BQ = 256, KS = DH / 16, NBLK = DH / 32;
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int fr = lane & 31, fg = lane >> 5;
+  // A workgroup takes query block nqblk-1-j of a (sequence, head) and then block j: under the causal mask block k costs
+  // k+1 units, so every workgroup costs the same (no longest-first dispatch, no tail), and the workgroups of one
+  // (sequence, head) start together and walk the key tiles of their long blocks in step.  They are also given to ONE
+  // XCD (workgroups are handed to the XCDs round robin), so that a K / V^T tile is fetched from memory once and found in
+  // that XCD's L2 by the others: fetched per query block from wherever it lies, the tiles were what bounded the kernel
+  // (1.2 GB per layer at 8 x 2048 tokens, ~5 TB/s).
+  const int nq2 = (nqblk + 1) / 2, npair = H * nseq;
+  int hb, j;
+  if (npair % 8 == 0) {
+    const int x = blockIdx.x & 7, r = blockIdx.x >> 3;
+    hb = (r / nq2) * 8 + x;
+    j = r % nq2;
+  } else {
+    hb = blockIdx.x % npair;
+    j = blockIdx.x / npair;
+  }
+  const int h = hb % H, b = hb / H;
+  const int64_t bh = (int64_t)b * H + h;
+  const float sc2 = rsqrtf((float)DH) * 1.4426950408889634f;   // 1/sqrt(dh) * log2(e): probabilities are 2^(s*sc2 - max)
+  const int nparts = (nqblk - 1 - j == j) ? 1 : 2;
+#pragma nounroll
+  for (int part = 0; part < nparts; ++part) {
+  const int qt0 = (part == 0 ? nqblk - 1 - j : j) * BQ;
+
+  // Q fragments of my two query blocks (B operand of S^T): lane (query fr, half fg) holds Q[t][ks*16 + fg*8 .. +8)
+  typename mma<T>::frag qf[2][KS];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int t = qt0 + wave * 64 + qb * 32 + fr;
+    const T* qp = q + (bh * Tp + (t < Tp ? t : Tp - 1)) * DH + fg * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[qb][ks] = mma<T>::load(qp + ks * 16);
+  }
+  const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(kc + bh * Tcap * DH), 0, (int)((int64_t)Tcap * DH * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(vt + bh * DH * ldvt), 0, (int)((int64_t)DH * ldvt * 2), 0x00020000);
+  // global -> LDS loads: a K tile is 16 wavefront loads of 2 rows (lane l fills position l % 32 of row 2j + l / 32 with
+  // chunk (p & 16) | ((p & 15) ^ (row & 15))), a V^T tile 16 loads of 16 rows (lane l fills position l % 4 of row
+  // 16j + l / 4 with chunk (l % 4) ^ ((row / 4) % 4)).  Wavefront w issues K loads j = 4jj + w and V^T loads j = 4w + jj,
+  // jj = 0 .. 3: the per-lane part of the address then depends on jj through one bit for K (row & 8) and not at all for
+  // V^T, and the rest is a scalar offset - three address registers instead of sixteen in a kernel that has none to spare.
+  const int k_row0 = 2 * wave + (lane >> 5);                                   // row of load jj: k_row0 + 8 jj
+  const int k_lo = k_row0 * 512 + (((lane & 16) | ((lane & 15) ^ (k_row0 & 15))) * 16);
+  const int v_lo = (int)((int64_t)(64 * wave + (lane >> 2)) * ldvt * 2) + (((lane & 3) ^ ((lane >> 4) & 3)) * 16);
+  const int v_step = (int)(ldvt * 32);                                         // 16 rows of V^T
+  auto issue_k1 = [&](int stage_tile, int tile, int jj) {
+    unsigned char* dst = smem + PP_LDS_K + (stage_tile & (PP_STAGES - 1)) * PP_KTILE + jj * 4096 + wave * 1024;
+    const int lo = (jj & 1) ? (k_lo ^ 128) : k_lo;
+    if (tile * BKV + BKV <= Tcap) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)dst, 16, lo, tile * (BKV * 512) + jj * 4096, 0, 0);
+    } else {      // rows beyond the window repeat its last row; their readers mask them
+      const int row = tile * BKV + k_row0 + 8 * jj;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr)dst, 16, (row < Tcap ? row : Tcap - 1) * 512 + (lo & 511), 0, 0, 0);
+    }
+  };
+  auto issue_v1 = [&](int stage_tile, int tile, int jj) {
+    const int col = (int64_t)tile * BKV + BKV <= ldvt ? tile * BKV : (int)ldvt - BKV;
+    unsigned char* dst = smem + PP_LDS_V + (stage_tile & (PP_STAGES - 1)) * PP_VTILE + wave * 4096 + jj * 1024;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr)dst, 16, v_lo, col * 2 + jj * v_step, 0, 0);
+  };
+  auto issue_k = [&](int stage_tile, int tile) {
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) issue_k1(stage_tile, tile, jj);
+  };
+  auto issue_v = [&](int stage_tile, int tile) {
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) issue_v1(stage_tile, tile, jj);
+  };
+  // tiles 0 .. 2 of K and 0 .. 1 of V^T go out before the sequence's padding is known (indices beyond the buffers are
+  // clamped into them; such a tile is never read)
+  issue_k(0, 0); issue_v(0, 0); issue_k(1, 1); issue_v(1, 1); issue_k(2, 2);
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) mma<T>::pin(qf[qb][ks]);   // pinned, or Q is re-loaded inside the key loop
+
+  const int p0 = pos0[b];                       // <= 0: minus the number of padding rows
+  const int klim = key_limit ? key_limit[b] : 0x7fffffff;
+  int qsee[2], wave_first[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int t = qt0 + wave * 64 + qb * 32 + fr;
+    const int qpos = (t < Tp) ? t + p0 : -1;    // this lane's position in block qb; < 0 = padding / out of range
+    qsee[qb] = qpos < klim ? qpos : klim;       // last key this query may see
+    const int wf0 = (qt0 + wave * 64 + qb * 32 + 31 < Tp) ? qt0 + wave * 64 + qb * 32 + p0 : -1;
+    wave_first[qb] = wf0 < klim ? wf0 : klim;   // a tile that ends at or below this needs no mask in block qb
+  }
+  const int last_t = (qt0 + BQ - 1 < Tp - 1) ? qt0 + BQ - 1 : Tp - 1;
+  const int kmax = last_t + p0;                 // last key any query of this workgroup may see
+  const int klast = Tp - 1 + p0;                // last key position that exists for this sequence
+  const int wave_last = qt0 + wave * 64 + 63 + p0;   // last key this wavefront may see
+  const int ntiles = (kmax >= 0) ? kmax / BKV + 1 : 0;
+  const int last = ntiles > 0 ? ntiles - 1 : 0;
+
+  // row fr of an S^T block is key krow: rows {0-3, 4-7, 8-11, 12-15} <- keys {0-3, 8-11, 4-7, 12-15} (+16)
+  const int krow = 16 * (fr >> 4) + 8 * ((fr >> 2) & 1) + 4 * ((fr >> 3) & 1) + (fr & 3);
+  const int kx = (krow & 15) ^ fg;              // chunk 2*ks + fg of row krow sits at ((2*(ks%8)) ^ kx) + 16*(ks/8)
+  const int kbase = krow * 512;
+  // worked out at every read: the score phase has vector-unit slots to spare, the register file has nothing
+  auto kxo = [&](int k) { return kbase + (((2 * k) ^ kx) << 4); };
+  const int vx = (fr >> 2) & 3;
+  const unsigned char* vbase = smem + PP_LDS_V + fr * 64;
+  const int vpos[2] = {((0 + fg) ^ vx) * 16, ((2 + fg) ^ vx) * 16};
+
+  acc_zero_all();                               // the output accumulator: a[0:255], see above
+  float mrun[2] = {-INFINITY, -INFINITY}, lrun[2] = {0.f, 0.f};
+  typename mma<T>::frag pf[2][2];               // probabilities of the previous tile: [query block][16-key half]
+  bool prev_active = false;
+
+  for (int i = 0; i <= ntiles; ++i) {
+    const int key0 = i * BKV;
+    // K tile i and V^T tile i-1 have landed once at most the 16 loads of the last two iterations are outstanding; the
+    // barrier also says that every wavefront is done with the stages that are requested next
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(16));
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    const int tk3 = i + 3 < last ? i + 3 : last, tv2 = i + 2 < last ? i + 2 : last;   // the tiles requested in this iteration
+    const bool active = i < ntiles && key0 <= wave_last;
+    floatx16 s[2];
+    if (active) {
+      // ---- scores of tile i: every K fragment feeds both query blocks
+      const unsigned char* kp = smem + PP_LDS_K + (i & (PP_STAGES - 1)) * PP_KTILE;
+      // with one wavefront per SIMD nothing but this wavefront's own earlier requests hides the LDS latency: the
+      // fragments of a pair of steps are requested while the pair before it multiplies (four matrix instructions)
+      typename mma<T>::frag kf[4];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) kf[j] = mma<T>::load(reinterpret_cast<const T*>(kp + kxo(j)));
+      // Two k-steps at a time, both into s[0], then both into s[1]: a matrix instruction whose accumulator is the
+      // result of the one right before it starts without delay (the result is forwarded), while one that accumulates
+      // onto the result of the instruction before last waits for the write-back - alternating s[0], s[1] per k-step
+      // ran at 50 cycles per instruction instead of 32.
+#pragma unroll
+      for (int ks = 0; ks < KS; ks += 2) {
+#pragma unroll
+        for (int d = 2; d < 4; ++d)
+          if (ks + d < KS)
+            kf[(ks + d) & 3] = mma<T>::load(reinterpret_cast<const T*>(kp + kxo((ks + d) & 7) + ((ks + d) >> 3) * 256));
+        // the eight global -> LDS requests of this iteration, one per pair of steps, under the matrix instructions
+        if (ks < 8) issue_k1(i + 3, tk3, ks / 2);
+        else issue_v1(i + 2, tv2, ks / 2 - 4);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks == 0) mma<T>::first_v(s[0], kf[0], qf[0][0]);
+        else mma<T>::run_v(s[0], kf[ks & 3], qf[0][ks]);
+        mma<T>::run_v(s[0], kf[(ks + 1) & 3], qf[0][ks + 1]);
+        if (ks == 0) mma<T>::first_v(s[1], kf[0], qf[1][0]);
+        else mma<T>::run_v(s[1], kf[ks & 3], qf[1][ks]);
+        mma<T>::run_v(s[1], kf[(ks + 1) & 3], qf[1][ks + 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");   // wait states between the last score MFMA and the first read of s
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        // register v is key key0 + 16*(v/8) + 8*fg + v%8
+        if (key0 + BKV - 1 > wave_first[qb]) {    // the diagonal crosses the tile: hide what a query may not see
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int key = key0 + 16 * (v / 8) + 8 * fg + (v % 8);
+            s[qb][v] = (key <= qsee[qb]) ? s[qb][v] : -INFINITY;
+          }
+        }
+      }
+    }
+    if (!active) {
+      issue_k(i + 3, tk3);
+      issue_v(i + 2, tv2);
+    }
+    if (prev_active) {
+      // the last tile of a sequence can be partial: what V^T holds beyond the last key must not reach the product
+      // (0 x garbage may be NaN).  Every wavefront clears all of it before its own reads (LDS operations of one
+      // wavefront stay in order), so no barrier is needed.
+      const int tv = i - 1;
+      const int nbad = tv * BKV + BKV - 1 - klast;
+      if (nbad > 0) {
+        uint16_t* vs = reinterpret_cast<uint16_t*>(smem + PP_LDS_V + (tv & (PP_STAGES - 1)) * PP_VTILE);
+        for (int c = lane; c < DH * nbad; c += 64) {
+          const int row = c / nbad, col = BKV - nbad + (c % nbad);
+          vs[row * 32 + (((col >> 3) ^ ((row >> 2) & 3)) * 8) + (col & 7)] = (uint16_t)0;
+        }
+      }
+    }
+    // ---- V^T P^T of tile i-1 on the matrix pipe with the exponentials of tile i on the vector unit between its
+    // instructions.  The exponentials are taken against the running maximum of the EARLIER tiles, so that nothing in
+    // this region waits for the maximum of tile i; that maximum is worked out alongside, and only if it lies more than
+    // 2^6 above the running one (probabilities would pass 64; after the first tiles it never does) the tile is redone
+    // below against the new maximum and the accumulator rescaled.
+    typename mma<T>::frag pn[2][2];
+    float mt[2] = {-INFINITY, -INFINITY}, lt[2] = {0.f, 0.f};
+    const float mneg[2] = {mrun[0] == -INFINITY ? 0.f : -mrun[0], mrun[1] == -INFINITY ? 0.f : -mrun[1]};
+    const unsigned char* vp = vbase + ((i - 1) & (PP_STAGES - 1)) * PP_VTILE;
+    float pe[2];                                  // the even-numbered probability of the pair being packed
+    auto exp_step = [&](auto K_) {                // step K of 32: probability K % 16 of query block K / 16
+      constexpr int k = decltype(K_)::value, qb = k / 16, v = k % 16;
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[qb][v], sc2, mneg[qb]));   // masked -> exp2(-inf) = 0
+      if constexpr (v % 2 == 0) {
+        pe[qb] = p;
+      } else {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        u32x4 w = __builtin_bit_cast(u32x4, pn[qb][v / 8].v);
+        w[(v % 8) / 2] = pack_prob<T>(pe[qb], p);
+        pn[qb][v / 8].v = __builtin_bit_cast(decltype(pn[qb][v / 8].v), w);
+      }
+      if constexpr (v % 4 == 3) mt[qb] = max3(max3(mt[qb], s[qb][v - 3], s[qb][v - 2]), s[qb][v - 1], s[qb][v]);
+      if constexpr (v % 8 == 7) lt[qb] = psum<T>::run(pn[qb][v / 8], lt[qb]);
+    };
+    __builtin_amdgcn_sched_barrier(0);
+    if (prev_active && active) {
+      typename mma<T>::frag vf[4];             // the V^T fragment of step j + 3 is requested while step j multiplies
+#pragma unroll
+      for (int j = 0; j < 3; ++j) vf[j] = mma<T>::load(reinterpret_cast<const T*>(vp + j * 2048 + vpos[0]));
+      static_for<16>([&](auto J_) {
+        constexpr int j = decltype(J_)::value, kh = j / 8, n = j % 8;
+        if constexpr (j + 3 < 16)
+          vf[(j + 3) & 3] = mma<T>::load(reinterpret_cast<const T*>(vp + ((j + 3) % 8) * 2048 + vpos[(j + 3) / 8]));
+        __builtin_amdgcn_sched_barrier(0);
+        mma<T>::template run_fixed<n * 16>(vf[j & 3], pf[0][kh]);
+        exp_step(std::integral_constant<int, 2 * j>{});
+        __builtin_amdgcn_sched_barrier(0);
+        mma<T>::template run_fixed<(8 + n) * 16>(vf[j & 3], pf[1][kh]);
+        exp_step(std::integral_constant<int, 2 * j + 1>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    } else if (prev_active) {
+      typename mma<T>::frag vf[4];
+#pragma unroll
+      for (int j = 0; j < 3; ++j) vf[j] = mma<T>::load(reinterpret_cast<const T*>(vp + j * 2048 + vpos[0]));
+      static_for<16>([&](auto J_) {
+        constexpr int j = decltype(J_)::value, kh = j / 8, n = j % 8;
+        if constexpr (j + 3 < 16)
+          vf[(j + 3) & 3] = mma<T>::load(reinterpret_cast<const T*>(vp + ((j + 3) % 8) * 2048 + vpos[(j + 3) / 8]));
+        __builtin_amdgcn_sched_barrier(0);
+        mma<T>::template run_fixed<n * 16>(vf[j & 3], pf[0][kh]);
+        mma<T>::template run_fixed<(8 + n) * 16>(vf[j & 3], pf[1][kh]);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    } else if (active) {
+      static_for<32>(exp_step);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (active) {
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        const float mtile = max_halves(mt[qb] * sc2);            // sc2 > 0
+        if (__any(mtile > mrun[qb] + 6.0f)) {
+          // rare: redo the tile against the new maximum and bring the accumulator (tiles 0 .. i-1) to it
+          const float mnew = fmaxf(mrun[qb], mtile);
+          const float alpha = (mnew == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(mrun[qb] - mnew);   // mrun = -inf -> 0
+          const float mn = (mnew == -INFINITY) ? 0.f : -mnew;
+          mrun[qb] = mnew;
+          float p[16];
+#pragma unroll
+          for (int v = 0; v < 16; ++v) p[v] = __builtin_amdgcn_exp2f(fmaf(s[qb][v], sc2, mn));
+          pn[qb][0] = mma<T>::from_floats(p);
+          pn[qb][1] = mma<T>::from_floats(p + 8);
+          lt[qb] = psum<T>::run(pn[qb][1], psum<T>::run(pn[qb][0], 0.f));
+          lrun[qb] *= alpha;
+          asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");     // the last MFMA into the accumulator may still be in flight
+          if (qb == 0) static_for<NBLK>([&](auto N_) { acc_scale16<decltype(N_)::value * 16>(alpha); });
+          else static_for<NBLK>([&](auto N_) { acc_scale16<(8 + decltype(N_)::value) * 16>(alpha); });
+        }
+        lrun[qb] += sum_halves(lt[qb]);
+        pf[qb][0] = pn[qb][0];
+        pf[qb][1] = pn[qb][1];
+      }
+    }
+    prev_active = active;
+  }
+  asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");           // the last MFMAs into the accumulator drain
+  // ---- write O.  Register v of block n is head-dim n*32 + 8*(v/4) + 4*fg + v%4 of the lane's query: stored from
+  // there, a store instruction would put 16 bytes into each of 32 rows.  The tiles are done with, so every wavefront
+  // turns its 64 rows round in its own 32 KiB of LDS (16-byte chunks xor-swizzled with the row) and writes whole rows.
+  __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));                // my surplus loads have landed ...
+  __builtin_amdgcn_s_barrier();                             // ... and so have everybody's; nobody reads a tile any more
+  unsigned char* ob = smem + wave * 32768;
+  static_for<2>([&](auto QB_) {
+    constexpr int qb = decltype(QB_)::value;
+    const int t = qt0 + wave * 64 + qb * 32 + fr;
+    const float inv = (t < Tp && t + p0 >= 0 && lrun[qb] > 0.f) ? 1.0f / lrun[qb] : 0.f;
+    static_for<NBLK * 4>([&](auto I_) {
+      constexpr int c = decltype(I_)::value, r = (qb * 8 + c / 4) * 16 + (c % 4) * 4;   // c: 16-byte chunk n*4 + v4 of the row
+      uint32x2 pk;
+      pk.x = pack2<T>(acc_read<r>() * inv, acc_read<r + 1>() * inv);
+      pk.y = pack2<T>(acc_read<r + 2>() * inv, acc_read<r + 3>() * inv);
+      *reinterpret_cast<uint32x2*>(ob + (qb * 32 + fr) * 512 + ((c ^ fr) << 4) + fg * 8) = pk;
+    });
+  });
+  // (a wavefront's LDS operations stay in order: no barrier between its own writes and reads)
+#pragma unroll 4
+  for (int it = 0; it < 32; ++it) {
+    const int row = 2 * it + fg, t = qt0 + wave * 64 + row;
+    const uint32x4 v = *reinterpret_cast<const uint32x4*>(ob + row * 512 + ((fr ^ (row & 31)) << 4));
+    if (t < Tp) *reinterpret_cast<uint32x4*>(out + ((int64_t)b * Tp + t) * ld_out + (int64_t)h * DH + fr * 8) = v;
+  }
+  __builtin_amdgcn_s_barrier();                             // the next part's tiles go where these rows were
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Decode.  Grid (S, H, B): the valid part of a (sequence, head) window is cut into S equal key ranges (the cut
 // follows the position read from device memory, so every workgroup has work whatever the fill), and each
 // 4-wavefront workgroup reduces its range to a partial (max, sum, weighted V).  A wavefront owns every fourth
@@ -875,7 +1274,25 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
         (const T*)q, (const T*)k_cache, (const T*)v_t, pos0, (int)H, (int)Tp, (int)Tcap, ldvt, (T*)out, ld_out,      \
         (int)B, (int)nqblk, key_limit);                                                                              \
   } while (0)
-  if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL_PAIR(bf16_t);
+#define MTJ_PREFILL_Q64(T)                                                                                           \
+  do {                                                                                                               \
+    static_assert(Q64_LDS_BYTES <= 160 * 1024, "attention tiles do not fit LDS");                                    \
+    static mtj_device_once once;                                                                                     \
+    if (int rc = mtj_allow_lds(once, "mtj_attn_prefill", &attn_prefill_q64_kernel<T>, Q64_LDS_BYTES)) return rc;     \
+    const int64_t nqblk = (Tp + 255) / 256;                                                                          \
+    MTJ_REQUIRE(nqblk * H * B < (1ll << 31), MTJ_ELIMIT, "mtj_attn_prefill: too many workgroups");                    \
+    MTJ_REQUIRE(Tcap * 512 < (1ll << 31) && 512 * ldvt < (1ll << 31), MTJ_ELIMIT, "mtj_attn_prefill: window too long"); \
+    attn_prefill_q64_kernel<T><<<(unsigned)((nqblk + 1) / 2 * H * B), 256, Q64_LDS_BYTES, s>>>(                                 \
+        (const T*)q, (const T*)k_cache, (const T*)v_t, pos0, (int)H, (int)Tp, (int)Tcap, ldvt, (T*)out, ld_out,      \
+        (int)B, (int)nqblk, key_limit);                                                                              \
+  } while (0)
+  // 256-query blocks, two per workgroup, when that still makes two workgroups per CU (measured on 16 heads x 2048 tokens:
+  // 472 us against 529 for 8 sequences, 796 against 1069 for 16, but 225 against 208 for 4); shorter problems keep the
+  // 128-query workgroups
+  const bool q64 = dh == 256 && B * H * ((Tp + 255) / 256) >= 1024;
+  if (dtype == MTJ_BF16 && q64) MTJ_PREFILL_Q64(bf16_t);
+  else if (dtype == MTJ_F16 && q64) MTJ_PREFILL_Q64(f16_t);
+  else if (dtype == MTJ_BF16 && dh == 256) MTJ_PREFILL_PAIR(bf16_t);
   else if (dtype == MTJ_BF16 && dh == 64) MTJ_PREFILL(bf16_t, 64, 8, 64);
   else if (dtype == MTJ_F16 && dh == 256) MTJ_PREFILL_PAIR(f16_t);
   else if (dtype == MTJ_F16 && dh == 64) MTJ_PREFILL(f16_t, 64, 8, 64);
@@ -884,6 +1301,7 @@ extern "C" int mtj_attn_prefill(const void* q, const void* k_cache, const void* 
   else return mtj_fail(MTJ_EINVAL, "mtj_attn_prefill: unsupported dtype %d / d_head %lld (64 or 256)", dtype, (long long)dh);
 #undef MTJ_PREFILL
 #undef MTJ_PREFILL_PAIR
+#undef MTJ_PREFILL_Q64
   return mtj_check_launch("mtj_attn_prefill");
 }
 
@@ -989,7 +1407,13 @@ int scratch_address(void** p) {
 }
 }  // namespace
 
-extern "C" int64_t mtj_attn_decode_static_max_bytes(void) { return MTJ_ATTN_DECODE_STATIC_BYTES; }
+// Also the set-up call: it looks the array's address up on the current device (a symbol lookup may load the code object
+// and must not happen inside a stream capture), so that mtj_attn_decode_static itself only launches.
+extern "C" int64_t mtj_attn_decode_static_max_bytes(void) {
+  void* p = nullptr;
+  (void)scratch_address(&p);          // without a usable device the size is still the answer; the entry point reports it
+  return MTJ_ATTN_DECODE_STATIC_BYTES;
+}
 
 extern "C" int mtj_attn_decode_static(const float* q, const void* k_cache, const void* v_cache, const int32_t* pos,
                                       int64_t B, int64_t H, int64_t Tcap, int64_t dh, void* out, int64_t ld_out,

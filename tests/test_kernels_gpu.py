@@ -556,6 +556,81 @@ def test_attn_prefill_full_context_d256(L, dt):
         assert float(row_err.max()) < 4 * ATT_TOL[dt], (dt, b, int(row_err.argmax()))
 
 
+def _attn_all_heads_f32(q, kk, vv, pads, key_limit=None):
+    """Every (sequence, head) at once in float32 on the GPU: a plain torch evaluation of the same masked softmax, for
+    shapes where the float64 host reference is only affordable on a few heads."""
+    B, H, Tp, dh = q.shape
+    sc = torch.einsum("bhtd,bhTd->bhtT", q.float(), kk.float()) / math.sqrt(dh)
+    idx = torch.arange(Tp, device=q.device)
+    hide = idx[None, :] > idx[:, None]                                  # causal
+    hide = hide[None] | (idx[None, None, :] < torch.tensor(pads, device=q.device)[:, None, None])
+    if key_limit is not None:
+        hide = hide | (idx[None, None, :] > torch.tensor(key_limit, device=q.device)[:, None, None])
+    sc = sc.masked_fill(hide[:, None], float("-inf"))
+    out = torch.einsum("bhtT,bhTd->bthd", torch.softmax(sc, -1), vv.float())
+    return out.reshape(B, Tp, H * dh)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("B,H,Tp,with_limit", [(64, 16, 200, False), (32, 16, 257, True), (128, 8, 33, False),
+                                               (8, 16, 2048, False), (11, 16, 1500, True), (35, 10, 700, False)])
+def test_attn_prefill_256_query_workgroups(L, dt, B, H, Tp, with_limit):
+    """Shapes with at least 1024 blocks of 256 queries run the kernel in which one wavefront owns 64 queries (d_head
+    256) and a workgroup two query blocks: ragged left padding per sequence, a query count that is no multiple of
+    anything, a partial last key tile (unwritten V^T columns are NaN), the evaluation key limit, the full 2048-token
+    context, an odd number of query blocks (the middle one has no partner), a number of (sequence, head) pairs that is
+    no multiple of 8.  Against the float64 reference on four (sequence, head) pairs and a float32 torch evaluation on
+    all of them."""
+    a = abi()
+    g = torch.Generator().manual_seed(B * 1000 + Tp)
+    dh = 256
+    assert B * H * ((Tp + 255) // 256) >= 1024
+    Tcap = Tp + 7
+    pads = [int(x) for x in torch.randint(0, max(min(Tp - 1, Tp // 3), 1), (B,), generator=g)]
+    pads[0] = 0
+    lim = [int(x) for x in torch.randint(Tp // 3, Tp, (B,), generator=g)] if with_limit else None
+    if with_limit:
+        pads = [0] * B                                              # the evaluation path has no padding
+    ldvt = (Tp + 63) // 64 * 64
+    q = torch.randn(B, H, Tp, dh, generator=g).to(TD[dt]).to(DEV)
+    kk = torch.randn(B, H, Tp, dh, generator=g).to(TD[dt]).to(DEV)
+    vv = torch.randn(B, H, Tp, dh, generator=g).to(TD[dt]).to(DEV)
+    kc = torch.zeros(B, H, Tcap, dh, dtype=TD[dt], device=DEV)
+    vt = torch.full((B, H, dh, ldvt), float("nan"), dtype=TD[dt], device=DEV)   # unwritten keys must never be read
+    for b in range(B):
+        n = Tp - pads[b]
+        kc[b, :, :n] = kk[b, :, pads[b]:]
+        vt[b, :, :, :n] = vv[b, :, pads[b]:].permute(0, 2, 1)
+    pos0 = torch.tensor([-pd for pd in pads], dtype=torch.int32, device=DEV)
+    kl = torch.tensor(lim, dtype=torch.int32, device=DEV) if with_limit else None
+    ld_out = H * dh + 8
+    out = torch.full((B * Tp, ld_out), 7.0, dtype=TD[dt], device=DEV)
+    a.check(L.mtj_attn_prefill(a.ptr(q), a.ptr(kc), a.ptr(vt), a.ptr(pos0), B, H, Tp, Tcap, dh, ldvt, a.ptr(out), ld_out,
+                               a.dtype_code(TD[dt]), a.ptr(kl), S()))
+    torch.cuda.synchronize()
+    assert torch.all(out[:, H * dh:] == 7.0)
+    got = out[:, :H * dh].reshape(B, Tp, H * dh).float()
+    assert bool(torch.isfinite(got).all())
+    ref32 = _attn_all_heads_f32(q, kk, vv, pads, lim)
+    for b in range(B):
+        pd = pads[b]
+        if pd:
+            assert float(got[b, :pd].abs().max()) == 0.0            # padding rows: zeros
+        e = float((got[b, pd:] - ref32[b, pd:]).norm() / ref32[b, pd:].norm())
+        assert e < ATT_TOL[dt], (dt, b, e)
+        row = (got[b, pd:] - ref32[b, pd:]).norm(dim=1) / ref32[b, pd:].norm(dim=1)
+        assert float(row.max()) < 6 * ATT_TOL[dt], (dt, b, int(row.argmax()) + pd)
+    for b, h in ((0, 0), (1, H - 1), (B - 1, H // 2), (B // 2, 3)):
+        qq, kq, vq = (t[b, h].double().cpu() for t in (q, kk, vv))
+        sc = qq @ kq.T / math.sqrt(dh)
+        idx = torch.arange(Tp)
+        hide = (idx[None, :] > idx[:, None]) | (idx[None, :] < pads[b])
+        if with_limit:
+            hide = hide | (idx[None, :] > lim[b])
+        ref = torch.softmax(sc.masked_fill(hide, float("-inf")), -1) @ vq
+        assert rel_err(got[b, pads[b]:, h * dh:(h + 1) * dh], ref[pads[b]:]) < ATT_TOL[dt], (dt, b, h)
+
+
 @pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("dh,H", [(64, 8), (256, 16)])
 @pytest.mark.parametrize("Tcap,positions", [(7, [0, 6, 9]), (300, [0, 150, 299]), (2047, [511, 2046, 5000]), (2047, [700]),

@@ -65,3 +65,41 @@ def test_static_scratch_rejects_oversize():
     assert b"built-in" in L.mtj_last_error()
     with pytest.raises(ValueError):
         a.check(rc)
+
+
+def test_static_scratch_under_graph_capture():
+    """The entry point is meant for captured code: after the set-up call and one eager call, a captured call must
+    replay to the bits of the eager workspace variant - several replays, with the inputs rewritten (by ordinary
+    eager work) between them."""
+    from mesh_transformer import _abi as a
+    L = a.lib()
+    assert L.mtj_attn_decode_static_max_bytes() > 0             # resolves the array's address on this device
+    B, H, Tcap, dh = 2, 16, 300, 256
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, H, dh, generator=g).to(DEV)
+    kc = torch.randn(B, H, Tcap, dh, generator=g).to(torch.float16).to(DEV)
+    vc = torch.randn(B, H, Tcap, dh, generator=g).to(torch.float16).to(DEV)
+    pos = torch.tensor([10, 250], dtype=torch.int32, device=DEV)
+    work = torch.zeros(L.mtj_attn_decode_work_bytes(B, H, dh, Tcap), dtype=torch.uint8, device=DEV)
+    ld = H * dh
+    out, ref = torch.zeros(B, ld, device=DEV), torch.zeros(B, ld, device=DEV)
+    dt = a.dtype_code(torch.float16)
+
+    def static_call():
+        a.check(L.mtj_attn_decode_static(a.ptr(q), a.ptr(kc), a.ptr(vc), a.ptr(pos), B, H, Tcap, dh, a.ptr(out), ld, 0, dt,
+                                         torch.cuda.current_stream().cuda_stream))
+
+    static_call()                                               # eager once: kernel attributes
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_call()
+    for rep, positions in enumerate(([10, 250], [299, 0], [150, 700])):
+        pos.copy_(torch.tensor(positions, dtype=torch.int32))
+        q.copy_(torch.randn(B, H, dh, generator=g))
+        out.fill_(float("nan"))
+        graph.replay()
+        a.check(L.mtj_attn_decode(a.ptr(q), a.ptr(kc), a.ptr(vc), a.ptr(pos), B, H, Tcap, dh, a.ptr(ref), ld, 0, dt,
+                                  a.ptr(work), torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref), (rep, float((out - ref).abs().max()))

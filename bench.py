@@ -34,7 +34,7 @@ for p in (ROOT, os.path.join(ROOT, "mesh-transformer-jax_amd")):
 HBM_PEAK = 8.0e12          # B/s
 # HBM bytes of one launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what
 # the same counter reads for a plain 234,881,024-byte copy (profiles/gemv_inproj_hbm_traffic_pmc.md)
-DOMINANT_KERNEL_TRAFFIC = 235603535
+DOMINANT_KERNEL_TRAFFIC = 235603296
 MFMA_BF16_PEAK = 2.5e15    # flop/s dense
 
 CFG_6B = dict(layers=28, d_model=4096, n_heads=16, n_vocab=50400, norm="layernorm", pe="rotary", pe_rotary_dims=64,
@@ -271,6 +271,10 @@ def main():
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter probe for rocprofv3 --pmc: one plain 234,881,024-byte device copy, then 8 launches "
                          "of the dominant kernel on a 2-layer model of the 6B shape; prints no JSON")
+    ap.add_argument("--decode-b32-probe", nargs=2, type=int, metavar=("PROMPT", "STEPS"),
+                    help="profiling probe: BASELINE config 4 (batch 32, nucleus sampling) with PROMPT-token prompts padded to "
+                         "2048 and STEPS decode steps, twice (the second run replays the recorded graphs); prints ms/step, "
+                         "no bench line")
     ap.add_argument("--prefill-probe", action="store_true",
                     help="profiling probe: 6 forwards of one full-shape layer on 8 x 2048 tokens (BASELINE config 2) "
                          "on a 1-layer model of the 6B shape; prints the time per forward, no bench line")
@@ -290,6 +294,20 @@ def main():
     dev = torch.device("cuda:0")
     if args.pmc_probe:
         pmc_probe(dev)
+        return
+    if args.decode_b32_probe:
+        P, G = args.decode_b32_probe
+        cfg = dict(CFG_6B, sampler=sampling.nucleaus_sample)
+        net = CausalTransformer(cfg, synthetic_tree(cfg, 2, dev, torch.bfloat16))
+        B, L = 32, 2048
+        u = np.random.Generator(np.random.Philox(3)).random((B, G))
+        ctx = O.left_pad(O.seeded_prompt(3, B, P), L)
+        opts = {"top_p": np.full(B, 0.9), "temp": np.full(B, 0.8)}
+        net.generate(ctx, np.full(B, P), G, opts, uniforms=u)
+        tm = {"warmup": 1}
+        net.generate(ctx, np.full(B, P), G, opts, uniforms=u, timing=tm)
+        print(json.dumps({"decode_b32_ms_per_step": tm["decode_s"] * 1e3 / tm["decode_steps"], "prompt": P, "steps": G,
+                          "keys": [P, P + G - 1]}))
         return
     if args.prefill_probe:
         c1 = dict(CFG_6B, layers=1, sampler=sampling.greedy_sample)

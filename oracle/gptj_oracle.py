@@ -146,6 +146,48 @@ def hashed_params(cfg, seed: int, weight_dtype=torch.bfloat16, std: float = 0.02
     return out
 
 
+def add_outliers(tree, cfg, gains=(0.5, 2.0, 0.5, 2.0)):
+    """Turns a synthetic tree into one shaped like a trained model, in place and with the SAME bits on any device: every
+    new value is a small integer pattern that bfloat16 holds exactly, every rescaling a power of two.  Four residual
+    channels carry +-50 .. +-500 from the embedding bias on and grow by a quarter of that through every fc_out bias;
+    LayerNorm scales run from 0.5 to 30 in steps of 0.5 (1 on the outlier channels) with offsets in [-0.5, 0.5]; the
+    rows of q, v, k and fc_in are divided by 1, 2 or 4 where the scale is below 2, 8 or 32 (and multiplied by `gains`,
+    powers of two, as whole matrices), the embedding matrix by 32; one k matrix holds +-4 next to its small entries."""
+    d, n = cfg["d_model"], cfg["layers"]
+    dev = tree[EMBED]["w"].device
+    c = torch.arange(d, device=dev)
+    ch = torch.tensor([7, 300, 511, 900], device=dev)
+    big = torch.tensor([300.0, -500.0, 50.0, -120.0], device=dev)
+    dt = tree[EMBED]["w"].dtype
+
+    def put(leaf, value):                                 # value float32 -> the leaf's dtype, one rounding
+        leaf.copy_(value.to(dt))
+
+    put(tree[EMBED]["w"], tree[EMBED]["w"].float() * 32.0)
+    b = tree[EMBED]["b"].float()
+    b[0, ch] = big
+    put(tree[EMBED]["b"], b)
+    for i in range(n):
+        sc = 0.5 + ((c * 37 + i * 11) % 60).float() * 0.5
+        sc[ch] = 1.0
+        off = (((c * 53 + i * 7) % 17).float() - 8.0) / 16.0
+        ln = tree[layer_key(i, "replicated_layer_norm")]
+        put(ln["scale"], sc[None])
+        put(ln["offset"], off[None])
+        b2 = tree[layer_key(i, "linear_5")]["b"].float()
+        b2[0, ch] += big * 0.25
+        put(tree[layer_key(i, "linear_5")]["b"], b2)
+        row = torch.where(sc < 2.0, 1.0, torch.where(sc < 8.0, 0.5, 0.25))       # per input channel
+        for name, gain in zip(("linear", "linear_1", "linear_2", "linear_4"), gains):
+            w = tree[layer_key(i, name)]["w"]
+            put(w, w.float() * (row * gain)[None, :, None])
+    w = tree[layer_key(min(1, n - 1), "linear_2")]["w"]
+    w[0, 5, 17], w[0, 700, 333] = 4.0, -4.0
+    put(tree[PROJ_LN]["scale"], (0.5 + ((c * 29) % 6).float() * 0.5)[None])
+    put(tree[PROJ_LN]["offset"], ((((c * 31) % 9).float() - 4.0) / 16.0)[None])
+    return tree
+
+
 def seeded_prompt(seed: int, batch: int, n: int, hi: int = 50257) -> np.ndarray:
     rng = np.random.Generator(np.random.Philox(seed + 1000003))
     return rng.integers(0, hi, size=(batch, n), dtype=np.int64).astype(np.uint32)

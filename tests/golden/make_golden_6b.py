@@ -4,12 +4,14 @@ tree (oracle.gptj_oracle.hashed_params), i.e. the reference's jnp.dot(f32, bf16)
   gptj6b_decode.npz    512-token prompt left-padded to 576, 32 greedy steps: tokens, top-32 / every 50th logit per step
   gptj6b_forward.npz   every-position logits of a 128-token forward (top-32 / every 50th logit per position)
   gptj6b_batch2.npz    two prompts (100 and 128 tokens, padded to 144), 8 greedy steps each
+  gptj6b_outlier_forward.npz   the 128-token forward on the same tree after oracle.gptj_oracle.add_outliers (residual
+                       channels of +-50 .. +-500 that grow with depth, LayerNorm scales up to 30, an entry of 4 in a k matrix)
 
 Greedy runs look for a prompt whose every greedy choice is decided by a clear margin (a near-tie would make the stream,
 and all logits after it, depend on rounding): the prefill is shared and only the last prompt token is varied.  The
 top-1/top-2 margin of every step is stored, so a test knows up to which step a free-running stream is decided.
 Needs ~45 GB of host memory and a quarter of an hour on 8 cores; run from the repository root:
-    python tests/golden/make_golden_6b.py [decode] [forward] [batch2]"""
+    python tests/golden/make_golden_6b.py [decode] [forward] [batch2] [outlier]"""
 import os
 import sys
 import time
@@ -127,6 +129,17 @@ def make_forward(model):
                         target_margin=target_margin, **summary(lg))
 
 
+def make_outlier_forward(model):
+    T = 128
+    prompt = O.seeded_prompt(5, 1, T)[0]
+    taps = []
+    lg = model.forward(prompt, taps).to(torch.float32).numpy()
+    log("outlier forward logits", lg.shape, "std", float(lg.std()), "absmax", float(np.abs(lg).max()),
+        "residual absmax per layer", [round(float(t.abs().max())) for t in taps])
+    np.savez_compressed(os.path.join(OUT, "gptj6b_outlier_forward.npz"), seed=SEED, ctx=prompt[None].astype(np.uint32),
+                        resid_absmax=np.asarray([float(t.abs().max()) for t in taps]), **summary(lg))
+
+
 def make_batch2(model):
     lens, L, G = [100, 128], 144, 8
     ctxs, toks, rows, margins = [], [], [], []
@@ -148,7 +161,18 @@ def make_batch2(model):
 
 
 def main():
-    what = sys.argv[1:] or ["decode", "forward", "batch2"]
+    what = sys.argv[1:] or ["decode", "forward", "batch2", "outlier"]
+    if "outlier" in what:
+        tree = O.add_outliers(O.hashed_params(CFG_6B, SEED, torch.bfloat16), CFG_6B)
+        log("outlier tree built")
+        model = O.Model(CFG_6B, tree, torch.float32)
+        del tree
+        with torch.no_grad():
+            make_outlier_forward(model)
+        del model
+        if what == ["outlier"]:
+            log("done")
+            return
     tree = O.hashed_params(CFG_6B, SEED, torch.bfloat16)
     log("tree built")
     model = O.Model(CFG_6B, tree, torch.float32)

@@ -277,3 +277,33 @@ def test_config2_one_full_shape_layer_against_the_float32_reference_layer():
         assert float(row.max()) < 4e-3, int(row.argmax())
     del eng
     torch.cuda.empty_cache()
+
+
+def test_outlier_channels_against_the_6b_oracle():
+    """The full 6B shape on a tree shaped like a trained model (oracle.gptj_oracle.add_outliers: residual channels of
+    +-50 .. +-500 that pass 3000 by the last layer, LayerNorm scales up to 30, an entry of 4 in a k matrix): the
+    every-position logits of a 128-token forward - float16 matrix-core operands end to end - and the logits of a
+    batch-1 decode step on the same tokens (float32 activations against bf16 weights) within 2e-2 of the oracle's
+    float32 run (tests/golden/gptj6b_outlier_forward.npz)."""
+    from oracle import gptj_oracle as O
+    from mesh_transformer import sampling
+    from mesh_transformer.transformer_shard import CausalTransformer
+    g = golden("gptj6b_outlier_forward.npz")
+    dev = torch.device("cuda:0")
+    tree = O.add_outliers(O.hashed_params(CFG_6B, int(g["seed"]), torch.bfloat16, device=dev), CFG_6B)
+    net = CausalTransformer(dict(CFG_6B, sampler=sampling.greedy_sample), tree)
+    ctx = g["ctx"]
+    lg = net.forward(ctx)[0].cpu().numpy()
+    e1, e2 = logit_errors(lg, g)
+    print("6B outlier tree, forward, 128 positions, vs the oracle: max |dlogit| strided", e1, "top-32", e2,
+          "; residual stream reaches", float(g["resid_absmax"].max()), "; logits std", float(g["strided_logits"].std()))
+    assert e1 < TOL_6B and e2 < TOL_6B
+    # the last position again through the decode path: prefill of 127 tokens, one decode step (left-padded, so that the
+    # window holds all 128 tokens)
+    _, out = net.generate(O.left_pad(ctx, 144), [ctx.shape[1]], 1, {}, return_logits=True)
+    last = {k: (g[k][-1:] if k in ("strided_logits", "top_ids", "top_logits") else g[k]) for k in g.files}
+    d1, d2 = logit_errors(out[2][0, :, 0], last)
+    print("6B outlier tree, decode step on the last token: max |dlogit| strided", d1, "top-32", d2)
+    assert d1 < TOL_6B and d2 < TOL_6B
+    del net
+    torch.cuda.empty_cache()

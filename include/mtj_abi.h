@@ -276,7 +276,11 @@ int mtj_sample_greedy(const float* logits, int64_t B, int64_t V, int32_t* tok, i
  * exp(filtered/temp - max) in float64 and the first token whose running weight exceeds u * total.
  * top_p, temp: float64 [B]; top_k: int32 [B] or NULL; uniforms: float64 [B, ld_u], column = step index.
  * keep_mask (optional) uint8 [B, V]: 1 where the filter left the logit untouched.
- * filtered (optional) float32 [B, V]: the filter's output.  `work` needs mtj_sample_work_bytes(B, V). */
+ * filtered (optional) float32 [B, V]: the filter's output.
+ * One launch, one workgroup per row; the row is not sorted: the rank at which a running sum crosses its threshold is
+ * found by selection, with the float64 weights accumulated exactly as 96-bit integers of 2^-62 (a decision differs
+ * from a sequential float64 running sum only if that sum lies within 1.4e-14 of the threshold).  V <= 65536.
+ * `work` (256-byte aligned, mtj_sample_work_bytes(B, V) = 256 bytes) is kept in the signature and not used. */
 int64_t mtj_sample_work_bytes(int64_t B, int64_t V);
 int mtj_sample_nucleus(const float* logits, int64_t B, int64_t V, const double* top_p, const double* temp,
                        const int32_t* top_k, const double* uniforms, int64_t ld_u, int32_t* tok,

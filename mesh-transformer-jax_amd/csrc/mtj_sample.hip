@@ -1,7 +1,6 @@
 // Samplers: greedy argmax, and nucleus (top-k / top-p) filtering with an inverse-CDF draw.
 #include <cstring>
 #include "mtj_common.h"
-#include <rocprim/device/device_merge_sort.hpp>
 
 namespace {
 
@@ -82,20 +81,6 @@ __device__ __forceinline__ float key_value(uint64_t k) {
   return __uint_as_float(u);
 }
 
-// All rows are sorted by one device-wide sort (a sort per row would leave most of the chip idle): bits 48..62
-// carry B-1-row, so that descending order keeps row 0 first and row b occupies [b*V, (b+1)*V) of the output.
-__global__ void make_keys_kernel(const float* __restrict__ logits, int64_t total, int V, int B, uint64_t* __restrict__ keys) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < total) {
-    const int64_t row = i / V;
-    keys[i] = ((uint64_t)(B - 1 - row) << 48) | sort_key(logits[i], (uint32_t)(i - row * V));
-  }
-}
-
-struct key_desc {
-  __device__ __forceinline__ bool operator()(const uint64_t& a, const uint64_t& b) const { return a > b; }
-};
-
 // f - a*b with the product rounded to float32 first (no fused multiply-add): logits -= 1e10 * mask is
 // two array operations in the reference (sampling.py:24-26)
 __device__ __forceinline__ float sub_product(float f, float a, float b) {
@@ -104,20 +89,305 @@ __device__ __forceinline__ float sub_product(float f, float a, float b) {
   return f - p;
 }
 
-// block-wide helpers (double)
-__device__ double block_sum(double v, double* sh) {
+// The sampler never sorts a row.  Both of its questions - where does the running softmax mass first exceed top_p,
+// and which token does u * total land on - ask for the first rank of the descending order at which a running
+// sum of non-negative weights exceeds a threshold, and so does top_k with unit weights.  Each is answered by
+// selection: a histogram of the weights over 4096 buckets that respect the order, a scan for the bucket where the
+// running sum crosses, and then the exact key among the few tokens of that bucket.
+// Weights are accumulated as integers (the float64 weight, at most 1, times 2^62, in 96 bits): integer sums do not
+// depend on the order of the atomic adds, so a row gives the same token on every run, and the sum of a bucket is
+// exactly the sum of its members, so the crossing found in the histogram is always found again inside the bucket.
+// A weight below 2^-62 counts as 0; a sum over 65536 tokens is therefore within 2^-46 of the float64 one, the same
+// order as the rounding of a sequential float64 sum.
+namespace sel {
+constexpr int NB = 4096;         // buckets per pass
+constexpr int LIST_CAP = 1024;   // keys of the crossing bucket kept in LDS
+constexpr double Q_ZERO = -43.0; // exp(t) * 2^62 < 1 below this
+
+struct acc {                     // 96-bit unsigned
+  uint64_t lo;
+  uint32_t hi;
+};
+__device__ __forceinline__ acc add(acc a, acc b) {
+  acc r;
+  r.lo = a.lo + b.lo;
+  r.hi = a.hi + b.hi + (r.lo < a.lo ? 1u : 0u);
+  return r;
+}
+__device__ __forceinline__ bool gt(acc a, acc b) { return a.hi != b.hi ? a.hi > b.hi : a.lo > b.lo; }
+__device__ __forceinline__ double to_double(acc a) { return (double)a.hi * 0x1p64 + (double)a.lo; }
+__device__ __forceinline__ acc from_double(double d) {   // 0 <= d < 2^96
+  acc r;
+  r.hi = (uint32_t)(d * 0x1p-64);
+  r.lo = (uint64_t)(d - (double)r.hi * 0x1p64);
+  return r;
+}
+// Copies the compiler knows nothing about: what one pass derives from a logit (its key, its bucket, whether its
+// token exists) is computed again in the next pass instead of being kept - fifty of each per thread would not fit
+// the register file.
+__device__ __forceinline__ float opaque(float x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+__device__ __forceinline__ int opaque(int x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+// A constant the compiler has to keep in scalar registers (it would otherwise copy it into vector registers
+// in front of every multiply-add that uses it).
+__device__ __forceinline__ double scalar_const(double c) {
+  asm volatile("" : "+s"(c));
+  return c;
+}
+// floor(exp(t) * 2^62) for -43 <= t <= 0, as the integer weight of a token: t = k ln 2 + r with |r| <= ln 2 / 2, the
+// Taylor polynomial of degree 13 for exp(r) (truncation error (ln 2 / 2)^14 / 14! = 4e-18), scaled by 2^(k + 62).
+struct exp_q {
+  double log2e, ln2_hi, ln2_lo, c[12];
+  __device__ __forceinline__ exp_q() {
+    log2e = scalar_const(0x1.71547652b82fep+0);
+    ln2_hi = scalar_const(-0x1.62e42fefa39efp-1);
+    ln2_lo = scalar_const(-0x1.abc9e3b39803fp-56);
+    double f = 1.0;
+    for (int i = 0; i < 12; ++i) {            // c[i] = 1 / (i + 2)!
+      f *= (double)(i + 2);
+      c[i] = scalar_const(1.0 / f);
+    }
+  }
+  __device__ __forceinline__ uint64_t operator()(double t) const {
+    const double kd = __builtin_rint(t * log2e);
+    double r = __builtin_fma(kd, ln2_hi, t);
+    r = __builtin_fma(kd, ln2_lo, r);
+    double p = c[11];
+#pragma unroll
+    for (int i = 10; i >= 0; --i) p = __builtin_fma(r, p, c[i]);
+    p = __builtin_fma(r, p, 1.0);
+    p = __builtin_fma(r, p, 1.0);
+    return (uint64_t)__builtin_ldexp(p, (int)kd + 62);
+  }
+};
+
+struct smem {
+  uint64_t ha[NB];               // per bucket: sum of the weights' bits 32 and up ...
+  uint64_t hb[NB];               // ... and of their low 32 bits (neither can overflow: no carry to pass on)
+  uint64_t list[LIST_CAP];
+  uint64_t wave_lo[SNT / 64];
+  uint32_t wave_hi[SNT / 64];
+  float fsh[SNT / 64];
+  uint64_t above_lo;
+  uint64_t key;
+  uint32_t above_hi;
+  int digit;
+  int n_list;
+  int hit;
+};
+
+// Bucket of pass 0: the distance below the row maximum in units of 1/scale, descending bucket = descending value.
+// Any weakly monotone function of the value would do; scale spreads the part of the row that can carry weight
+// over all buckets (the high bits of the float would put half of a row in two or three).
+__device__ __forceinline__ int coarse(float l, float l0, float scale) {
+  const int c = (int)fminf((l0 - l) * scale, (float)(NB - 1));   // NaN -> NB-1
+  return NB - 1 - max(c, 0);
+}
+__device__ __forceinline__ float coarse_scale(float range) { return (float)(NB - 1) / range; }
+
+template <bool COUNT>
+__device__ __forceinline__ void hist_add(smem& S, int b, uint64_t q) {
+  if (!COUNT) atomicAdd(reinterpret_cast<unsigned long long*>(&S.ha[b]), (unsigned long long)(q >> 32));
+  atomicAdd(reinterpret_cast<unsigned long long*>(&S.hb[b]), (unsigned long long)(q & 0xffffffffull));
+}
+__device__ __forceinline__ acc bucket(const smem& S, int b) {
+  const uint64_t a = S.ha[b], c = S.hb[b];
+  acc r;
+  r.lo = (a << 32) + c;
+  r.hi = (uint32_t)(a >> 32) + (r.lo < c ? 1u : 0u);
+  return r;
+}
+
+struct scan_t {
+  acc s[4];      // running sums over this thread's four buckets, in descending bucket order
+  acc before;    // sum of the buckets ahead of them
+  acc grand;     // sum of all buckets
+};
+// thread t owns buckets NB-1-4t .. NB-4-4t
+__device__ __forceinline__ scan_t scan_hist(smem& S) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  scan_t r;
+  acc run{0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    run = add(run, bucket(S, NB - 1 - (4 * tid + j)));
+    r.s[j] = run;
+  }
+  acc inc = run;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    acc t;
+    t.lo = __shfl_up((unsigned long long)inc.lo, o);
+    t.hi = __shfl_up(inc.hi, o);
+    if (lane >= o) inc = add(inc, t);
+  }
+  acc ex;
+  ex.lo = __shfl_up((unsigned long long)inc.lo, 1);
+  ex.hi = __shfl_up(inc.hi, 1);
+  if (lane == 0) ex = acc{0, 0};
+  if (lane == 63) { S.wave_lo[wave] = inc.lo; S.wave_hi[wave] = inc.hi; }
+  __syncthreads();
+  acc base{0, 0}, grand{0, 0};
+  for (int w = 0; w < SNT / 64; ++w) {
+    const acc t{S.wave_lo[w], S.wave_hi[w]};
+    if (w < wave) base = add(base, t);
+    grand = add(grand, t);
+  }
+  r.before = add(base, ex);
+  r.grand = grand;
+  return r;
+}
+// The bucket in which `above` + running sum first exceeds T, if any: returns its index (-1: none) and moves `above`
+// to the sum ahead of it.  All threads return the same answer.
+__device__ __forceinline__ int pick(smem& S, const scan_t& sc, acc& above, acc T) {
+  const int tid = threadIdx.x;
+  const acc base = add(above, sc.before);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const acc excl = j ? add(base, sc.s[j - 1]) : base;
+    const acc incl = add(base, sc.s[j]);
+    if (!gt(excl, T) && gt(incl, T)) {
+      S.digit = NB - 1 - (4 * tid + j);
+      S.above_lo = excl.lo;
+      S.above_hi = excl.hi;
+    }
+  }
+  __syncthreads();
+  const int d = S.digit;
+  if (d >= 0) above = acc{S.above_lo, S.above_hi};
+  __syncthreads();
+  return d;
+}
+__device__ __forceinline__ void clear_hist(smem& S) {
+  for (int i = threadIdx.x; i < NB; i += SNT) { S.ha[i] = 0; S.hb[i] = 0; }
+  if (threadIdx.x == 0) { S.digit = -1; S.hit = 0; }
+}
+__device__ __forceinline__ uint64_t readlane_u64(uint64_t v, int j) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, j);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), j);
+  return ((uint64_t)hi << 32) | lo;
+}
+
+// First key of the descending order at which the running sum of wq(l, id, key) exceeds thr(total) (a double in the
+// same 2^-62 units; negative: the first key with a weight; NaN or no crossing: returns false).  l0 is the row
+// maximum, scale the bucket width of pass 0.  COUNT: the weights are 0 or 1.
+template <int NT_MAX, bool COUNT, class WQ, class THR>
+__device__ __forceinline__ bool select(smem& S, const float (&l)[NT_MAX], int V, float l0, float scale, WQ wq, THR thr,
+                                       uint64_t& key_out) {
+  const int tid = threadIdx.x;
+  // ---- pass 0: every token of the row into its bucket
+  clear_hist(S);
+  if (tid == 0) S.n_list = 0;
+  __syncthreads();
+#pragma unroll
+  for (int n = 0; n < NT_MAX; ++n) {
+    const int id = opaque(tid) + n * SNT;
+    if (id < V) {
+      const float x = opaque(l[n]);
+      const uint64_t q = wq(x, (uint32_t)id, sort_key(x, (uint32_t)id));
+      if (q) hist_add<COUNT>(S, coarse(x, l0, scale), q);
+    }
+    __builtin_amdgcn_sched_barrier(0);   // one token at a time: fifty exponentials in flight would spill
+  }
+  __syncthreads();
+  scan_t sc = scan_hist(S);
+  const double td = thr(to_double(sc.grand));
+  if (!(td < 0x1p95)) return false;               // NaN or beyond any sum (every thread has the same td)
+  const acc T = td > 0.0 ? from_double(td) : acc{0, 0};
+  acc above{0, 0};
+  const int g = pick(S, sc, above, T);
+  if (g < 0) return false;
+  // ---- the keys of that bucket go to LDS if they fit
+#pragma unroll
+  for (int n = 0; n < NT_MAX; ++n) {
+    const int id = opaque(tid) + n * SNT;
+    const float x = opaque(l[n]);
+    if (id < V && coarse(x, l0, scale) == g) {
+      const int at = atomicAdd(&S.n_list, 1);
+      if (at < LIST_CAP) S.list[at] = sort_key(x, (uint32_t)id);
+    }
+  }
+  __syncthreads();
+  const int n_list = __builtin_amdgcn_readfirstlane(S.n_list);
+  if (n_list <= 64) {
+    // ---- one wavefront, one key per lane: the sum ahead of a key is the sum over the keys above it
+    if (tid < 64) {
+      uint64_t key = 0, q = 0;
+      if (tid < n_list) {
+        key = S.list[tid];
+        q = wq(key_value(key), (uint32_t)(key & 0xffffu), key);
+      }
+      acc ahead = above;
+      for (int j = 0; j < n_list; ++j) {
+        const uint64_t kj = readlane_u64(key, j), qj = readlane_u64(q, j);
+        const acc t = add(ahead, acc{qj, 0});
+        if (kj > key) ahead = t;
+      }
+      if (tid < n_list && !gt(ahead, T) && gt(add(ahead, acc{q, 0}), T)) { S.key = key; S.hit = 1; }
+    }
+    __syncthreads();
+    if (!S.hit) return false;                     // cannot happen: the sums are exact
+    key_out = S.key;
+    __syncthreads();
+    return true;
+  }
+  // ---- a crowded bucket (many equal or nearly equal logits): four 12-bit digits of the key inside it
+  uint64_t prefix = 0;
+  for (int d = 1; d <= 4; ++d) {
+    const int shift = 48 - 12 * d;
+    clear_hist(S);
+    __syncthreads();
+    if (n_list <= LIST_CAP) {
+      for (int i = tid; i < n_list; i += SNT) {
+        const uint64_t key = S.list[i];
+        if ((key >> (shift + 12)) == prefix) {
+          const uint64_t q = wq(key_value(key), (uint32_t)(key & 0xffffu), key);
+          if (q) hist_add<COUNT>(S, (int)((key >> shift) & (NB - 1)), q);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int n = 0; n < NT_MAX; ++n) {
+        const int id = opaque(tid) + n * SNT;
+        const float x = opaque(l[n]);
+        if (id < V && coarse(x, l0, scale) == g) {
+          const uint64_t key = sort_key(x, (uint32_t)id);
+          if ((key >> (shift + 12)) == prefix) {
+            const uint64_t q = wq(x, (uint32_t)id, key);
+            if (q) hist_add<COUNT>(S, (int)((key >> shift) & (NB - 1)), q);
+          }
+        }
+      }
+    }
+    __syncthreads();
+    sc = scan_hist(S);
+    const int dg = pick(S, sc, above, T);
+    if (dg < 0) return false;                     // cannot happen: the sums are exact
+    prefix = (prefix << 12) | (uint64_t)dg;
+  }
+  key_out = prefix;
+  return true;
+}
+
+__device__ __forceinline__ float block_max_f(smem& S, float v) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
   __syncthreads();
-  if (lane == 0) sh[wave] = v;
+  if (lane == 0) S.fsh[wave] = v;
   __syncthreads();
-  double t = 0.0;
-  for (int w = 0; w < SNT / 64; ++w) t += sh[w];
+  float t = S.fsh[0];
+  for (int w = 1; w < SNT / 64; ++w) t = fmaxf(t, S.fsh[w]);
   return t;
 }
-__device__ double block_max(double v, double* sh) {
+__device__ __forceinline__ double block_max_d(smem& S, double v) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  double* sh = reinterpret_cast<double*>(S.wave_lo);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v = fmax(v, __shfl_xor(v, o));
   __syncthreads();
@@ -127,187 +397,155 @@ __device__ double block_max(double v, double* sh) {
   for (int w = 1; w < SNT / 64; ++w) t = fmax(t, sh[w]);
   return t;
 }
-// exclusive prefix over per-thread totals, in thread order
-__device__ double block_exclusive(double v, double* sh) {
+// minimum (want_max = false) or maximum of a 64-bit key over the workgroup
+__device__ __forceinline__ uint64_t block_ext_u64(smem& S, uint64_t v, bool want_max) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  double inc = v;
 #pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const double t = __shfl_up(inc, o);
-    if (lane >= o) inc += t;
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint64_t t = __shfl_xor((unsigned long long)v, o);
+    v = want_max ? (t > v ? t : v) : (t < v ? t : v);
   }
   __syncthreads();
-  if (lane == 63) sh[wave] = inc;
+  if (lane == 0) S.wave_lo[wave] = v;
   __syncthreads();
-  double base = 0.0;
-  for (int w = 0; w < wave; ++w) base += sh[w];
-  return base + inc - v;
+  uint64_t r = S.wave_lo[0];
+  for (int w = 1; w < SNT / 64; ++w) r = want_max ? (S.wave_lo[w] > r ? S.wave_lo[w] : r) : (S.wave_lo[w] < r ? S.wave_lo[w] : r);
+  return r;
 }
+}  // namespace sel
 
-// wave-wide inclusive prefix sum (double), lanes in order
-__device__ __forceinline__ double wave_inclusive(double v) {
-  const int lane = threadIdx.x & 63;
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const double t = __shfl_up(v, o);
-    if (lane >= o) v += t;
-  }
-  return v;
-}
+constexpr size_t SEL_LDS_BYTES = sizeof(sel::smem);
 
-// One workgroup of 16 wavefronts per row.  Wavefront w owns ranks [w*NT*64, (w+1)*NT*64) of the sorted order in
-// NT tiles of 64 consecutive ranks (lane = rank inside the tile: coalesced reads); the sorted values and ids
-// stay in registers for all three sweeps, and running sums are carried tile to tile inside the wavefront.
-template <int NT_MAX>        // tiles per wavefront: V <= 16 * 64 * NT_MAX
-__global__ __launch_bounds__(SNT) void nucleus_kernel(const float* __restrict__ logits, const uint64_t* __restrict__ sorted,
-                                                      int V, const double* __restrict__ top_p,
-                                                      const double* __restrict__ temp, const int32_t* __restrict__ top_k,
+// One workgroup of 1024 threads per row; thread t keeps tokens t, t + 1024, ... in registers for every pass.
+template <int NT_MAX>        // tokens per thread: V <= 1024 * NT_MAX
+__global__ __launch_bounds__(SNT) void nucleus_kernel(const float* __restrict__ logits, int V,
+                                                      const double* __restrict__ top_p, const double* __restrict__ temp,
+                                                      const int32_t* __restrict__ top_k,
                                                       const double* __restrict__ uniforms, int64_t ld_u,
                                                       int32_t* __restrict__ tok, int32_t* __restrict__ out_tokens,
                                                       int64_t ld_tokens, int32_t* __restrict__ pos,
                                                       const int32_t* __restrict__ pos_start,
                                                       uint8_t* __restrict__ keep_mask, float* __restrict__ filtered,
                                                       const mtj_next_embed ne) {
-  __shared__ double sh[SNT / 64];
-  __shared__ int sh_i[SNT / 64];
-  __shared__ int chosen;
-  const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const uint64_t* srt = sorted + (int64_t)b * V;
-  const int nt = (V + SNT - 1) / SNT;             // tiles per wavefront (uniform), <= NT_MAX
-  const int jw = wave * nt * 64 + lane;           // my rank in tile 0
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  sel::smem& S = *reinterpret_cast<sel::smem*>(smem_raw);
+  const int b = blockIdx.x, tid = threadIdx.x;
+  const float* row = logits + (int64_t)b * V;
   const int step = pos[b] - pos_start[b];
   const double tp = top_p[b], tmp = temp[b], u = uniforms[(int64_t)b * ld_u + step];
   const int kk = top_k ? top_k[b] : 0x7fffffff;
 
-  float val[NT_MAX];                              // sorted logits of my ranks (-inf beyond V)
-  uint32_t idp[NT_MAX / 2];                       // their token ids, two per register
+  float l[NT_MAX];
 #pragma unroll
-  for (int t = 0; t < NT_MAX; ++t) {
-    val[t] = -INFINITY;
-    if ((t & 1) == 0) idp[t / 2] = 0;
-    if (t < nt) {
-      const int j = jw + t * 64;
-      if (j < V) {
-        const uint64_t key = srt[j];
-        val[t] = key_value(key);
-        idp[t / 2] |= (uint32_t)(key & 0xffffu) << (16 * (t & 1));
-      }
-    }
+  for (int n = 0; n < NT_MAX; ++n) l[n] = row[min(tid + n * SNT, V - 1)];     // all loads in flight together
+  float lmax = -INFINITY, lmin = INFINITY;
+#pragma unroll
+  for (int n = 0; n < NT_MAX; ++n) {
+    const bool live = tid + n * SNT < V;
+    lmin = fminf(lmin, live ? l[n] : INFINITY);
+    l[n] = live ? l[n] : -INFINITY;
+    lmax = fmaxf(lmax, l[n]);
   }
-  auto id_of = [&](int t) { return (idp[t / 2] >> (16 * (t & 1))) & 0xffffu; };
+  const float l0 = sel::block_max_f(S, lmax);
+  const float spread = l0 + sel::block_max_f(S, -lmin);      // row maximum - row minimum
+  const double l0d = (double)l0;
+  const sel::exp_q expq;
 
-  // ---- softmax of the sorted logits (the maximum is rank 0)
-  const double l0 = (double)key_value(srt[0]);
-  double loc = 0.0;
-#pragma unroll
-  for (int t = 0; t < NT_MAX; ++t)
-    if (t < nt) loc += (jw + t * 64 < V) ? exp((double)val[t] - l0) : 0.0;
-  const double Z = block_sum(loc, sh);            // leaves the per-wavefront sums in sh
-  double base = 0.0;                              // mass of the ranks before my wavefront's
-  for (int w = 0; w < wave; ++w) base += sh[w] / Z;
-  __syncthreads();
-
-  // ---- filter: remove rank j when the mass of ranks [0, j-1] already exceeds top_p (sampling.py:28-30)
-  uint64_t removed = 0;                           // bit t: my rank of tile t is outside the nucleus
-  double tmax = -INFINITY;
-  auto filtered_of = [&](int t, uint32_t id, float l) {
-    float f = l;
-    if (jw + t * 64 >= kk) f = sub_product(f, 1e10f, (float)id);   // top-k quirk: subtracts 1e10 * token id
-    return f - (((removed >> t) & 1) ? 1e10f : 0.0f);
+  // ---- top_p: rank j > 0 leaves the nucleus when the softmax mass of ranks [0, j-1] exceeds top_p (sampling.py:28-30),
+  // that is, every key below the one at which the running mass first exceeds it
+  uint64_t key_p = 0, key_k = 0;
+  const bool cut_p = sel::select<NT_MAX, false>(
+      S, l, V, l0, sel::coarse_scale(fminf(spread, 43.0f)),
+      [&](float x, uint32_t, uint64_t) {
+        const double t = (double)x - l0d;
+        return t < sel::Q_ZERO ? (uint64_t)0 : expq(t);
+      },
+      [&](double total) { return tp * total; }, key_p);
+  // ---- top_k: ranks >= top_k, every key below the one of rank top_k - 1
+  bool cut_k = false;
+  if (kk >= 1 && kk < V)
+    cut_k = sel::select<NT_MAX, true>(
+        S, l, V, l0, sel::coarse_scale(fminf(spread, 1e4f)), [](float, uint32_t, uint64_t) { return (uint64_t)1; },
+        [&](double) { return (double)(kk - 1); }, key_k);
+  auto filtered_of = [&](float x, uint32_t id, uint64_t key) {
+    float f = x;
+    if (kk < 1 || (cut_k && key < key_k)) f = sub_product(f, 1e10f, (float)id);   // top-k quirk: subtracts 1e10 * token id
+    return f - ((cut_p && key < key_p) ? 1e10f : 0.0f);
   };
+
+  // ---- the filter's output, when asked for
+  if (filtered || keep_mask) {
 #pragma unroll
-  for (int t = 0; t < NT_MAX; ++t) {
-    if (t < nt) {
-      const int j = jw + t * 64;
-      const bool live = j < V;
-      if (base > tp) {
-        // the mass before this tile already exceeds top_p (base is the same in every lane, and it only grows):
-        // every rank of the tile is outside the nucleus, no exponential needed
-        if (live && j > 0) removed |= 1ull << t;
-      } else {
-        const double e = live ? exp((double)val[t] - l0) / Z : 0.0;
-        const double incl = wave_inclusive(e);
-        const double before = base + (incl - e);
-        if (live && j > 0 && before > tp) removed |= 1ull << t;
-        base += __shfl(incl, 63);
-      }
-      if (live) {
-        const uint32_t id = id_of(t);
-        // the sort key folds -0.0 into +0.0: fetch the original bits for a zero
-        const float l = (val[t] == 0.0f) ? logits[(int64_t)b * V + id] : val[t];
-        const float f = filtered_of(t, id, l);
+    for (int n = 0; n < NT_MAX; ++n) {
+      const int id = sel::opaque(tid) + n * SNT;
+      if (id < V) {
+        const float x = sel::opaque(l[n]);
+        const float f = filtered_of(x, (uint32_t)id, sort_key(x, (uint32_t)id));
         if (filtered) filtered[(int64_t)b * V + id] = f;
-        if (keep_mask) keep_mask[(int64_t)b * V + id] = (f == l) ? 1 : 0;
-        tmax = fmax(tmax, (double)f / tmp);
+        if (keep_mask) keep_mask[(int64_t)b * V + id] = (f == x) ? 1 : 0;
       }
     }
   }
-  tmax = block_max(tmax, sh);
-  // ---- inverse-CDF draw over exp(filtered / temp - max) in sorted order
-  // exp(x) is exactly 0 in float64 below -745.14: what the filter pushed down by 1e10 (almost every rank of a peaked
-  // distribution) needs no exponential
-  auto weight = [&](int t) {
-    const double x = (double)filtered_of(t, id_of(t), val[t]) / tmp - tmax;
-    return x < -746.0 ? 0.0 : exp(x);
-  };
-  double wloc = 0.0;
+  // ---- the largest filtered / temp
+  double tmax;
+  if (tmp > 0.0 && kk >= 1) {
+    // the filter only lowers a logit and leaves rank 0 alone, and x -> x / temp is monotone
+    tmax = l0d / tmp;
+  } else {                    // top_k < 1 penalises every rank, temp <= 0 or NaN turns the order around: token by token
+    double m = -INFINITY;
 #pragma unroll
-  for (int t = 0; t < NT_MAX; ++t)
-    if (t < nt && jw + t * 64 < V) wloc += weight(t);
-  const double total = block_sum(wloc, sh);
-  double cum = 0.0;
-  for (int w = 0; w < wave; ++w) cum += sh[w];
-  const double target = u * total;
-  int first = 0x7fffffff, lastpos = -1;
-#pragma unroll
-  for (int t = 0; t < NT_MAX; ++t) {
-    if (t < nt) {
-      const int j = jw + t * 64;
-      const double w = (j < V) ? weight(t) : 0.0;
-      const double incl = wave_inclusive(w);
-      if (w > 0.0) lastpos = j;
-      if (cum + incl > target && j < V && first == 0x7fffffff) first = j;
-      cum += __shfl(incl, 63);
+    for (int n = 0; n < NT_MAX; ++n) {
+      const int id = sel::opaque(tid) + n * SNT;
+      const float x = sel::opaque(l[n]);
+      if (id < V) m = fmax(m, (double)filtered_of(x, (uint32_t)id, sort_key(x, (uint32_t)id)) / tmp);
     }
+    tmax = sel::block_max_d(S, m);
   }
-  // min over first, max over lastpos
+
+  // ---- inverse-CDF draw over exp(filtered / temp - max) in descending order of the raw logits
+  // In the usual case a token the filter touched has no weight at all (its filtered / temp is 1e10 / temp lower,
+  // far below the 2^-62 that still counts) and needs no arithmetic; token 0 is exempt from the top-k penalty, which
+  // multiplies by the token id.
+  const bool plain = tmp > 0.0 && tmp <= 1e6 && kk >= 1 && fabsf(l0) <= 1e6f;
+  uint64_t key_t = 0;
+  const bool hit = sel::select<NT_MAX, false>(
+      S, l, V, l0, sel::coarse_scale(fminf(spread, tmp > 0.0 ? (float)fmin(43.0 * fmax(tmp, 1.0), 1e30) : 1e30f)),
+      [&](float x, uint32_t id, uint64_t key) {
+        double t;
+        if (plain) {
+          if ((cut_p && key < key_p) || (cut_k && key < key_k && id != 0)) return (uint64_t)0;
+          t = (double)x / tmp - tmax;
+        } else {
+          t = (double)filtered_of(x, id, key) / tmp - tmax;
+        }
+        return (t < sel::Q_ZERO || !(t <= 0.0)) ? (uint64_t)0 : expq(t);
+      },
+      [&](double total) { return u * total; }, key_t);
+  if (!hit) {
+    // u * total is not exceeded: the last rank with a weight (exp(x) is exactly 0 in float64 below -745.14), else rank 0
+    uint64_t lowest = ~0ull, top = 0;
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    first = min(first, __shfl_xor(first, o));
-    lastpos = max(lastpos, __shfl_xor(lastpos, o));
+    for (int n = 0; n < NT_MAX; ++n) {
+      const int id = sel::opaque(tid) + n * SNT;
+      if (id < V) {
+        const float x = sel::opaque(l[n]);
+        const uint64_t key = sort_key(x, (uint32_t)id);
+        top = key > top ? key : top;
+        const double t = (double)filtered_of(x, (uint32_t)id, key) / tmp - tmax;
+        if (t >= -746.0 && exp(t) > 0.0) lowest = key < lowest ? key : lowest;
+      }
+    }
+    lowest = sel::block_ext_u64(S, lowest, false);
+    top = sel::block_ext_u64(S, top, true);
+    key_t = lowest != ~0ull ? lowest : top;
   }
-  __syncthreads();
-  if (lane == 0) { sh_i[wave] = first; sh[wave] = (double)lastpos; }
-  __syncthreads();
+  const int id = (int)(key_t & 0xffffu);
   if (tid == 0) {
-    int f = 0x7fffffff, lp = -1;
-    for (int w = 0; w < SNT / 64; ++w) { f = min(f, sh_i[w]); lp = max(lp, (int)sh[w]); }
-    int j = (f != 0x7fffffff) ? f : (lp >= 0 ? lp : 0);
-    const int id = (int)(srt[j] & 0xffffu);
     tok[b] = id;
     if (out_tokens) out_tokens[(int64_t)b * ld_tokens + step] = id;
     pos[b] += 1;
-    chosen = id;
   }
-  __syncthreads();
-  embed_next(ne, b, V, chosen);
-}
-
-struct sample_layout {
-  size_t keys_in, keys_out, sort_temp, total;
-};
-size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-
-// rocPRIM's merge sort needs one more buffer of keys plus a few words per block; a fixed upper bound, so that
-// the size query does not need a device.
-sample_layout layout(int64_t B, int64_t V) {
-  sample_layout L;
-  size_t o = 0;
-  L.keys_in = o;  o += align256((size_t)B * V * 8);
-  L.keys_out = o; o += align256((size_t)B * V * 8);
-  L.sort_temp = o; o += align256((size_t)B * V * 8 + (size_t)B * 64 + (1 << 16));
-  L.total = o;
-  return L;
+  embed_next(ne, b, V, id);
 }
 
 }  // namespace
@@ -332,7 +570,11 @@ extern "C" int mtj_sample_greedy(const float* logits, int64_t B, int64_t V, int3
   return mtj_check_launch("mtj_sample_greedy");
 }
 
-extern "C" int64_t mtj_sample_work_bytes(int64_t B, int64_t V) { return (int64_t)layout(B, V).total; }
+// The selection kernel keeps everything in registers and LDS; the work buffer of the ABI is not used by it.
+extern "C" int64_t mtj_sample_work_bytes(int64_t B, int64_t V) {
+  (void)B; (void)V;
+  return 256;
+}
 
 extern "C" int mtj_sample_nucleus(const float* logits, int64_t B, int64_t V, const double* top_p, const double* temp,
                                   const int32_t* top_k, const double* uniforms, int64_t ld_u, int32_t* tok,
@@ -347,24 +589,14 @@ extern "C" int mtj_sample_nucleus(const float* logits, int64_t B, int64_t V, con
   mtj_next_embed ne;
   if (int rc = check_next(next, &ne, "mtj_sample_nucleus")) return rc;
   hipStream_t s = (hipStream_t)stream;
-  const sample_layout L = layout(B, V);
-  unsigned char* w = reinterpret_cast<unsigned char*>(work);
-  uint64_t* kin = reinterpret_cast<uint64_t*>(w + L.keys_in);
-  uint64_t* kout = reinterpret_cast<uint64_t*>(w + L.keys_out);
-  const int64_t total = B * V;
-  make_keys_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(logits, total, (int)V, (int)B, kin);
-  size_t need = 0;
-  hipError_t e = rocprim::merge_sort(nullptr, need, kin, kout, (size_t)total, key_desc(), s, false);
-  if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_sample_nucleus: sort size query: %s", hipGetErrorString(e));
-  const size_t have = L.total - L.sort_temp;
-  MTJ_REQUIRE(need <= have, MTJ_ELIMIT, "mtj_sample_nucleus: sort scratch %zu > reserved %zu", need, have);
-  e = rocprim::merge_sort(w + L.sort_temp, need, kin, kout, (size_t)total, key_desc(), s, false);
-  if (e != hipSuccess) return mtj_fail(MTJ_EHIP, "mtj_sample_nucleus: sort: %s", hipGetErrorString(e));
-  if (V <= SNT * 50)      // GPT-J's 50400-entry vocabulary: everything stays in registers
-    nucleus_kernel<50><<<(unsigned)B, SNT, 0, s>>>(logits, kout, (int)V, top_p, temp, top_k, uniforms, ld_u, tok, out_tokens,
+  static mtj_device_once once50, once64;
+  if (int rc = mtj_allow_lds(once50, "mtj_sample_nucleus", &nucleus_kernel<50>, SEL_LDS_BYTES)) return rc;
+  if (int rc = mtj_allow_lds(once64, "mtj_sample_nucleus", &nucleus_kernel<64>, SEL_LDS_BYTES)) return rc;
+  if (V <= SNT * 50)      // GPT-J's 50400-entry vocabulary
+    nucleus_kernel<50><<<(unsigned)B, SNT, SEL_LDS_BYTES, s>>>(logits, (int)V, top_p, temp, top_k, uniforms, ld_u, tok, out_tokens,
                                                    ld_tokens, pos, pos_start, keep_mask, filtered, ne);
   else
-    nucleus_kernel<64><<<(unsigned)B, SNT, 0, s>>>(logits, kout, (int)V, top_p, temp, top_k, uniforms, ld_u, tok, out_tokens,
+    nucleus_kernel<64><<<(unsigned)B, SNT, SEL_LDS_BYTES, s>>>(logits, (int)V, top_p, temp, top_k, uniforms, ld_u, tok, out_tokens,
                                                    ld_tokens, pos, pos_start, keep_mask, filtered, ne);
   return mtj_check_launch("mtj_sample_nucleus");
 }

@@ -64,7 +64,7 @@ def test_argument_validation_needs_no_device():
     assert lib.mtj_attn_decode_splits(1, 16, 2047) == 8 and lib.mtj_attn_decode_splits(32, 16, 2047) == 1
     assert lib.mtj_attn_decode_splits(1, 16, 20) == 2          # never fewer than 16 slots per range at a full window
     assert lib.mtj_attn_decode_work_bytes(1, 16, 256, 2047) == 16 * 8 * 260 * 4
-    assert lib.mtj_sample_work_bytes(32, 50400) > 2 * 32 * 50400 * 8
+    assert lib.mtj_sample_work_bytes(32, 50400) == 256         # kept in the ABI; the sampler sorts nothing
 
 
 def test_host_tensors_are_refused():

@@ -844,6 +844,53 @@ def test_nucleus_bit_exact_vs_oracle(L, V, spread):
             assert tok[r] == O.inverse_cdf_draw(logits[r:r + 1], f_ref, float(temp[r]), float(u[r])), (V, spread, r, k)
 
 
+def _check_rows(L, logits, top_p, temp, top_k, u):
+    tok, mask, filt = _sample(L, logits, top_p, temp, top_k, u)
+    for r in range(logits.shape[0]):
+        k = None if top_k is None else int(np.broadcast_to(top_k, (logits.shape[0],))[r])
+        tp, tm, ur = (float(np.broadcast_to(v, (logits.shape[0],))[r]) for v in (top_p, temp, u))
+        f_ref = O.nucleaus_filter(logits[r:r + 1], tp, k)
+        assert np.array_equal(filt[r:r + 1], f_ref), r
+        assert np.array_equal(mask[r], f_ref[0] == logits[r]), r
+        assert tok[r] == O.inverse_cdf_draw(logits[r:r + 1], f_ref, tm, ur), r
+
+
+@pytest.mark.parametrize("V", [50400, 65536, 700])
+def test_nucleus_crowded_and_degenerate_rows(L, V):
+    """Rows that defeat the bucketing of the selection: every logit equal, hundreds of copies of the value at which
+    the running mass crosses, -inf entries, one far outlier, a row whose whole weight sits on one token."""
+    rng = np.random.default_rng(V)
+    R = 7
+    logits = (rng.standard_normal((R, V)) * 2.0).astype(np.float32)
+    logits[0] = 0.25                                        # one bucket, one value: ids decide
+    logits[1, rng.permutation(V)[: V // 3]] = logits[1].max()   # the mass crosses inside a run of equal maxima
+    logits[2, ::5] = -np.inf
+    logits[3, 17] = 3.0e5                                   # everything else has no weight
+    logits[4] = np.round(logits[4] * 4) / 4                 # 40-odd distinct values
+    logits[5, : V // 2] = -1.0e4
+    logits[6] = np.linspace(-3, 3, V, dtype=np.float32)[rng.permutation(V)]
+    top_p = np.array([0.9001, 0.5003, 0.9, 0.9, 0.8002, 0.95, 0.3001])
+    temp = np.array([1.0, 0.7, 1.3, 0.8, 1.0, 2.5, 0.05])
+    for u in (rng.random(R), np.zeros(R), np.full(R, 0.999999)):
+        _check_rows(L, logits, top_p, temp, None, u)
+    _check_rows(L, logits, top_p, temp, np.array([V // 2, 3, 1, 2, 100, V - 1, 64], np.int32), rng.random(R))
+
+
+def test_nucleus_unusual_parameters(L):
+    """Parameters outside the usual case, where a filtered token keeps a weight or the order of filtered / temp
+    turns around: top_k 0 (every rank penalised by 1e10 * id), temperatures of 1e8 and 1e10 (1e10 / temp is no longer
+    out of reach), u = 1 (no running weight exceeds the total: the last token with a weight), top_p 0 and below."""
+    rng = np.random.default_rng(11)
+    V, R = 3000, 6
+    logits = (rng.standard_normal((R, V)) * 1.5).astype(np.float32)
+    top_p = np.array([0.9, 0.6, 0.9, 0.0, -1.0, 0.7])
+    temp = np.array([1.0, 1e8, 1e10, 0.9, 1.1, 0.6])
+    u = np.array([0.3, 0.77, 0.52, 0.5, 0.5, 1.0])
+    _check_rows(L, logits, top_p, temp, None, u)
+    _check_rows(L, logits, top_p, temp, np.array([0, 10, 5, V, V + 7, 1], np.int32), u)
+    _check_rows(L, logits[:, :1].copy(), top_p, temp, None, u)          # a vocabulary of one
+
+
 def test_nucleus_against_the_committed_fixture(L):
     """tests/golden/nucleus_cases.npz: keep-masks and tokens bit for bit."""
     import os

@@ -142,8 +142,10 @@ def time_decode_b32(net, cfg, B=32, P=1024, L=2048, G=1024, tail=64):
     ctx = O.left_pad(O.seeded_prompt(3, B, P), L)
     opts = {"top_p": np.full(B, 0.9), "temp": np.full(B, 0.8)}
     tm = {"warmup": G - tail}
-    net.generate(ctx, np.full(B, P), G, opts, uniforms=u)             # untimed: allocates, records the graphs
-    net.generate(ctx, np.full(B, P), G, opts, uniforms=u, timing=tm)
+    from mesh_transformer import sampling
+    nucleus = sampling.nucleaus_sample                                # whatever sampler the net was configured with
+    net.generate(ctx, np.full(B, P), G, opts, uniforms=u, sampler=nucleus)   # untimed: allocates, records the graphs
+    net.generate(ctx, np.full(B, P), G, opts, uniforms=u, sampler=nucleus, timing=tm)
     net.engine().sessions.pop((B, L - 1), None)
 
     def leg(seconds, first, n):

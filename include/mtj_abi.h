@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define MTJ_ABI_VERSION 3
+#define MTJ_ABI_VERSION 4
 
 enum { MTJ_F32 = 0, MTJ_BF16 = 1, MTJ_F16 = 2 };
 
@@ -269,6 +269,18 @@ typedef struct {
 int mtj_sample_greedy(const float* logits, int64_t B, int64_t V, int32_t* tok, int32_t* out_tokens,
                       int64_t ld_tokens, int32_t* pos, const int32_t* pos_start, const mtj_next_embed* next,
                       void* stream);
+
+/* The logits projection of a batch-1 decode step and the greedy sampler behind it in one launch
+ * (transformer_shard.py:107-113 and :203): mtj_gemv with MTJ_EPI_STORE into float32 `logits` [N] followed by
+ * mtj_sample_greedy(logits, 1, N, ...), same results bit for bit.  Every workgroup folds the best of its rows into
+ * work[0] with a 64-bit atomic maximum and counts its arrival in work[128 bytes]; the workgroup that completes the
+ * count does the sampler's part (tok, out_tokens, pos += 1, x_next) and puts both words back to 0 - no workgroup waits
+ * for another.  `work`: 256 bytes, 256-byte aligned, zeroed once by the caller; launches that share it must not
+ * overlap in time. */
+int mtj_gemv_greedy(const float* x, const float* ln_scale, const float* ln_offset, const void* W, const float* bias,
+                    int64_t N, int64_t K, int dtype, float* logits, int32_t* tok, int32_t* out_tokens,
+                    int64_t ld_tokens, int32_t* pos, const int32_t* pos_start, const mtj_next_embed* next, void* work,
+                    void* stream);
 
 /* nucleaus_sample (sampling.py:10-44) with the Gumbel draw replaced by an inverse-CDF draw from
  * host-supplied uniforms: filter on the RAW logits (optional top_k, then top_p, float64 softmax and

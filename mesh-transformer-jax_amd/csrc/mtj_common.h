@@ -376,3 +376,17 @@ __device__ __forceinline__ void inproj_store(const mtj_inproj& ip, const float* 
                                              float own, float partner) {
   inproj_finish(ip, inproj_prepare(ip, b1, m, n), own, partner);
 }
+
+// x_next[b, :] = W[token, :] + bias by the whole workgroup (token is uniform): the embedding of the token a sampler
+// just chose (EmbeddingShard, layers.py:187-202), which is the input of the next decode step
+__device__ __forceinline__ void embed_next(const mtj_next_embed& ne, int b, int V, int token) {
+  if (!ne.w) return;
+  const bool hit = (uint32_t)token < (uint32_t)V;
+  float* xo = ne.x_next + (int64_t)b * ne.d;
+  for (int64_t c = threadIdx.x; c < ne.d; c += blockDim.x) {
+    float w = 0.f;
+    if (hit) w = ne.dtype == MTJ_F32 ? reinterpret_cast<const float*>(ne.w)[(int64_t)token * ne.d + c]
+                                     : elem<bf16_t>::load(reinterpret_cast<const bf16_t*>(ne.w) + (int64_t)token * ne.d + c);
+    xo[c] = w + ne.bias[c];
+  }
+}

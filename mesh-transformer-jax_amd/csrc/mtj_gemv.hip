@@ -60,6 +60,14 @@ struct gemv_args {
   mtj_inproj ip;
   mtj_attn_merge am;      // partials == NULL: x is read as it is
   int upb, upb_rem;       // units per workgroup: the first upb_rem workgroups take upb + 1 (set by launch())
+  // ARGMAX only: the greedy sampler behind a STORE of one row of logits
+  unsigned long long* am_work;   // [0] best (value image, ~index) so far, [16] arrivals; both 0 between launches
+  int32_t* tok;
+  int32_t* out_tokens;
+  int64_t ld_tokens;
+  int32_t* pos;
+  const int32_t* pos_start;
+  mtj_next_embed ne;
 };
 
 // Stages the input vector of a matrix-vector kernel into LDS: LayerNorm on the fly (two passes, as the reference
@@ -146,7 +154,13 @@ __device__ __forceinline__ void stage_x(const gemv_args& a, float* __restrict__ 
 // against 39.4 with the row sums routed through LDS so that one thread finishes a row and adjacent threads adjacent
 // rows; cutting the rows into 1 KiB pieces so that consecutive wavefronts read consecutive KiB takes 49.7 us.)
 // MERGE: the leading inputs are merged from one-token attention partials (a.am) instead of being read from x.
-template <typename T, int U, bool FULL, bool MERGE>
+// ARGMAX (with a STORE epilogue): the launch also is the greedy sampler of the row it writes.  Every workgroup folds
+// the best of its rows into one 64-bit word with an atomic maximum - the monotone image of the float above the
+// complement of the index, so that the largest value wins and among equal values the lowest index - and then counts
+// its arrival; the workgroup whose arrival completes the count reads the word, which by then holds every
+// workgroup's contribution, and does what the sampler does (token, position, embedding of the token for the next
+// step), and puts both words back to 0.  Nobody waits for anybody: the order in which workgroups run does not matter.
+template <typename T, int U, bool FULL, bool MERGE, bool ARGMAX = false>
 __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
   extern __shared__ __align__(16) float xs[];
   __shared__ float red[2][16];
@@ -278,9 +292,50 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const gemv_args a) {
     if (a.epi == MTJ_EPI_STORE) store_as(a.out, n, mine + pre_add, a.out_dtype);
     else reinterpret_cast<float*>(a.out)[n] = mine + pre_add;
   }
+  if constexpr (ARGMAX) {
+    __shared__ unsigned long long best_of_wave[16];
+    __shared__ int chosen;                                   // the token, in the workgroup that arrives last; else -1
+    unsigned long long best = 0;
+    if (lane < nrows) {
+      const float v = (mine + pre_add) + 0.0f;               // -0.0 -> +0.0: equal to it in a comparison
+      uint32_t u = __float_as_uint(v);
+      u = (v != v) ? 0u : ((u & 0x80000000u) ? ~u : (u | 0x80000000u));   // a NaN never wins
+      best = ((unsigned long long)u << 32) | (uint32_t)~(uint32_t)(row0 + lane);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const unsigned long long t = __shfl_xor(best, o);
+      best = t > best ? t : best;
+    }
+    if (lane == 0) best_of_wave[wave] = best;
+    if (tid == 0) chosen = -1;
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+      for (int w = 1; w < 16; ++w) best = best_of_wave[w] > best ? best_of_wave[w] : best;
+      unsigned long long seen =
+          __hip_atomic_fetch_max(a.am_work, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      asm volatile("" : "+v"(seen) : : "memory");            // the maximum is in place before the arrival is counted
+      const unsigned long long before =
+          __hip_atomic_fetch_add(a.am_work + 16, 1ull + (seen & 0ull), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (before == (unsigned long long)gridDim.x - 1) {
+        const unsigned long long all = __hip_atomic_load(a.am_work, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(a.am_work, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(a.am_work + 16, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int t = (int)(uint32_t)~(uint32_t)all;
+        if (t < 0 || t >= (int)a.N) t = 0;
+        a.tok[0] = t;
+        if (a.out_tokens) a.out_tokens[a.pos[0] - a.pos_start[0]] = t;
+        a.pos[0] += 1;
+        chosen = t;
+      }
+    }
+    __syncthreads();
+    if (chosen >= 0) embed_next(a.ne, 0, (int)a.N, chosen);
+  }
 }
 
-template <typename T, int U, bool FULL, bool MERGE>
+template <typename T, int U, bool FULL, bool MERGE, bool ARGMAX = false>
 int launch(const gemv_args& a, hipStream_t s) {
   const size_t lds = (size_t)a.K * sizeof(float);
   const int64_t units = a.epi == MTJ_EPI_INPROJ ? a.N / 2 : a.N;
@@ -290,11 +345,11 @@ int launch(const gemv_args& a, hipStream_t s) {
   const int64_t upw = a.epi == MTJ_EPI_INPROJ ? 2 : 1;
   while ((units + grid * 16 - 1) / (grid * 16) * upw > 62) grid *= 2;   // a lane per row: <= 64 rows per wavefront
   static mtj_device_once once;
-  if (int rc = mtj_allow_lds(once, "mtj_gemv", &gemv_kernel<T, U, FULL, MERGE>, 160 * 1024 - 256)) return rc;
+  if (int rc = mtj_allow_lds(once, "mtj_gemv", &gemv_kernel<T, U, FULL, MERGE, ARGMAX>, 160 * 1024 - 512)) return rc;
   gemv_args b = a;
   b.upb = (int)(units / grid);
   b.upb_rem = (int)(units % grid);
-  gemv_kernel<T, U, FULL, MERGE><<<(unsigned)grid, 1024, lds, s>>>(b);
+  gemv_kernel<T, U, FULL, MERGE, ARGMAX><<<(unsigned)grid, 1024, lds, s>>>(b);
   return mtj_check_launch("mtj_gemv");
 }
 
@@ -640,6 +695,7 @@ template <typename T>
 int dispatch(const gemv_args& a, hipStream_t s) {
   constexpr int U = 8;
   const bool full = a.K % (U * 64 * chunk<T>::EPC) == 0;
+  if (a.am_work) return full ? launch<T, U, true, false, true>(a, s) : launch<T, U, false, false, true>(a, s);
   if (a.am.partials) return full ? launch<T, U, true, true>(a, s) : launch<T, U, false, true>(a, s);
   return full ? launch<T, U, true, false>(a, s) : launch<T, U, false, false>(a, s);
 }
@@ -689,6 +745,35 @@ extern "C" int mtj_gemv(const float* x, const float* ln_scale, const float* ln_o
   if (dtype == MTJ_BF16) return dispatch<bf16_t>(a, s);
   if (dtype == MTJ_F16) return dispatch<f16_t>(a, s);
   return mtj_fail(MTJ_EDTYPE, "mtj_gemv: dtype %d", dtype);
+}
+
+extern "C" int mtj_gemv_greedy(const float* x, const float* ln_scale, const float* ln_offset, const void* W,
+                               const float* bias, int64_t N, int64_t K, int dtype, float* logits, int32_t* tok,
+                               int32_t* out_tokens, int64_t ld_tokens, int32_t* pos, const int32_t* pos_start,
+                               const mtj_next_embed* next, void* work, void* stream) {
+  MTJ_REQUIRE(x && W && logits && tok && pos && pos_start && work, MTJ_EINVAL, "mtj_gemv_greedy: null pointer");
+  MTJ_REQUIRE(N > 0 && N < (1ll << 31) && K > 0 && K % 8 == 0, MTJ_EINVAL,
+              "mtj_gemv_greedy: K=%lld must be a positive multiple of 8, N below 2^31", (long long)K);
+  MTJ_REQUIRE(K * 4 <= 160 * 1024 - 512, MTJ_ELIMIT, "mtj_gemv_greedy: K=%lld floats do not fit LDS", (long long)K);
+  MTJ_REQUIRE(mtj_aligned16(x) && mtj_aligned16(W), MTJ_EALIGN, "mtj_gemv_greedy: x and W must be 16-byte aligned");
+  MTJ_REQUIRE((reinterpret_cast<uintptr_t>(work) & 255u) == 0, MTJ_EALIGN, "mtj_gemv_greedy: work must be 256-byte aligned");
+  MTJ_REQUIRE((ln_scale == nullptr) == (ln_offset == nullptr), MTJ_EINVAL, "mtj_gemv_greedy: ln_scale/ln_offset go together");
+  gemv_args a{};
+  a.x = x; a.ln_scale = ln_scale; a.ln_offset = ln_offset; a.W = W; a.bias = bias;
+  a.N = N; a.K = K; a.epi = MTJ_EPI_STORE; a.out = logits; a.out_dtype = MTJ_F32;
+  a.am_work = reinterpret_cast<unsigned long long*>(work);
+  a.tok = tok; a.out_tokens = out_tokens; a.ld_tokens = ld_tokens; a.pos = pos; a.pos_start = pos_start;
+  a.ne = mtj_next_embed{nullptr, nullptr, nullptr, 0, 0};
+  if (next && next->w) {
+    MTJ_REQUIRE(next->bias && next->x_next && next->d > 0 && (next->dtype == MTJ_F32 || next->dtype == MTJ_BF16), MTJ_EINVAL,
+                "mtj_gemv_greedy: incomplete next-step embedding");
+    a.ne = *next;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == MTJ_F32) return dispatch<float>(a, s);
+  if (dtype == MTJ_BF16) return dispatch<bf16_t>(a, s);
+  if (dtype == MTJ_F16) return dispatch<f16_t>(a, s);
+  return mtj_fail(MTJ_EDTYPE, "mtj_gemv_greedy: dtype %d", dtype);
 }
 
 // ------------------------------------------------------------------------------------------------ fused out projection

@@ -6,19 +6,6 @@ namespace {
 
 constexpr int SNT = 1024;  // threads per row
 
-// x_next[b, :] = W[token, :] + bias, by the whole workgroup (token is uniform)
-__device__ __forceinline__ void embed_next(const mtj_next_embed& ne, int b, int V, int token) {
-  if (!ne.w) return;
-  const bool hit = (uint32_t)token < (uint32_t)V;
-  float* xo = ne.x_next + (int64_t)b * ne.d;
-  for (int64_t c = threadIdx.x; c < ne.d; c += blockDim.x) {
-    float w = 0.f;
-    if (hit) w = ne.dtype == MTJ_F32 ? reinterpret_cast<const float*>(ne.w)[(int64_t)token * ne.d + c]
-                                     : elem<bf16_t>::load(reinterpret_cast<const bf16_t*>(ne.w) + (int64_t)token * ne.d + c);
-    xo[c] = w + ne.bias[c];
-  }
-}
-
 // ---------------------------------------------------------------- greedy
 __global__ __launch_bounds__(SNT) void greedy_kernel(const float* __restrict__ logits, int V, int32_t* __restrict__ tok,
                                                      int32_t* __restrict__ out_tokens, int64_t ld_tokens,

@@ -9,7 +9,7 @@ import os
 
 F32, BF16, F16 = 0, 1, 2
 EPI_STORE, EPI_RESID, EPI_INPROJ = 0, 1, 2
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmtj_hip.so")
 
@@ -67,6 +67,7 @@ SIGNATURES = {
     "mtj_attn_decode_static_max_bytes": (_i64, []),
     "mtj_attn_decode_static": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _i64, _i32, _i32, _p]),
     "mtj_sample_greedy": (_i32, [_p, _i64, _i64, _p, _p, _i64, _p, _p, C.POINTER(NextEmbed), _p]),
+    "mtj_gemv_greedy": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _p, _p, _p, _i64, _p, _p, C.POINTER(NextEmbed), _p, _p]),
     "mtj_sample_work_bytes": (_i64, [_i64, _i64]),
     "mtj_sample_nucleus": (_i32, [_p, _i64, _i64, _p, _p, _p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p,
                                  C.POINTER(NextEmbed), _p]),

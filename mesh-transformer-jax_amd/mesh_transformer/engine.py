@@ -206,6 +206,9 @@ class Session:
                                L.mtj_gemv_attn_supported(d, d + F, w.dtype, H, dh, w.act_dtype, Tcap))
         self.oa_work = torch.zeros(L.mtj_gemv_attn_work_bytes(H, dh), dtype=torch.uint8, device=dev) if self.fused_attn else None
         self.sample_work = None
+        # best-so-far word and arrival counter of the logits launch that is its own greedy sampler (batch 1)
+        self.fused_greedy = bool(self.gemv_path and cfg.get("fused_greedy_sampler", True))
+        self.greedy_work = torch.zeros(256, dtype=torch.uint8, device=dev) if self.fused_greedy else None
         self.tok = torch.zeros(B, dtype=torch.int32, device=dev)
         self.pos = torch.zeros(B, dtype=torch.int32, device=dev)
         self.pos_start = torch.zeros(B, dtype=torch.int32, device=dev)
@@ -310,9 +313,11 @@ class Engine:
         ne.w, ne.bias, ne.x_next, ne.d, ne.dtype = ptr(w.we), ptr(w.be), ptr(ses.x), w.d, w.dtype
         return C.byref(ne)
 
-    def decode_model(self, ses, logits=None):
+    def decode_model(self, ses, logits=None, greedy_out=None, embed_next=True):
         """generate_once (transformer_shard.py:97-115) from the embedded token in ses.x to the logits (ses.logits, or
-        the [B, V] float32 tensor given); the K/V window is updated in place."""
+        the [B, V] float32 tensor given); the K/V window is updated in place.  With greedy_out (the [B, G] token
+        buffer) the batch-1 logits launch also is the greedy sampler - sample_greedy's effects are then already in
+        place and the call returns True; otherwise (batched decode) it returns False and the caller samples."""
         L, w, s = _abi.lib(), self.w, _abi.stream_handle()
         B, d, F, V = ses.B, w.d, w.F, w.V
         logits = ses.logits if logits is None else logits
@@ -326,9 +331,14 @@ class Engine:
                 self.layer_decode(ses, i, normed=True, next_ln=nxt)
             check(L.mtj_gemm(ptr(ses.h), d, ptr(w.w_p_mm), ptr(w.b_p), B, V, d, w.mm_dtype, EPI_STORE, ptr(logits), V,
                              F32, None, w.alpha_p, s))
-            return
+            return False
         for i in w.layer_ids:
             self.layer_decode(ses, i)
+        if ses.fused_greedy and greedy_out is not None:
+            check(L.mtj_gemv_greedy(ptr(ses.x), ptr(w.pln_s), ptr(w.pln_o), ptr(w.w_p), ptr(w.b_p), V, d, w.dtype,
+                                    ptr(logits), ptr(ses.tok), ptr(greedy_out), greedy_out.shape[1], ptr(ses.pos),
+                                    ptr(ses.pos_start), self._next(ses, embed_next), ptr(ses.greedy_work), s))
+            return True
         if ses.gemv_path:
             check(L.mtj_gemv(ptr(ses.x), ptr(w.pln_s), ptr(w.pln_o), ptr(w.w_p), ptr(w.b_p), V, d, w.dtype, EPI_STORE,
                              ptr(logits), F32, None, None, s))

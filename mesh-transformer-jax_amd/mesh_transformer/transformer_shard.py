@@ -105,7 +105,8 @@ class CausalTransformer:
     config keys read: layers, d_model, n_heads, n_vocab, norm, pe, pe_rotary_dims, cores_per_replica,
     sampler (callable, transformer_shard.py:191), early_cast.  Extra, optional: "device",
     "steps_per_graph" (decode steps recorded into one HIP graph, default 8; 0 disables graphs),
-    "fused_decode_attention" (batch-1 decode computes the attention inside the out-projection launch, default True)."""
+    "fused_decode_attention" (batch-1 decode computes the attention inside the out-projection launch, default True),
+    "fused_greedy_sampler" (batch-1 greedy decode takes the argmax inside the logits launch, default True)."""
 
     def __init__(self, config, params=None):
         self.config = config
@@ -344,10 +345,11 @@ class CausalTransformer:
             ses.graphs = {}
 
     def _step(self, eng, ses, kind, keep_mask=None, logits=None):
-        eng.decode_model(ses, logits)
         if kind == "greedy":
-            eng.sample_greedy(ses, ses.out_tokens, logits=logits)
+            if not eng.decode_model(ses, logits, greedy_out=ses.out_tokens):
+                eng.sample_greedy(ses, ses.out_tokens, logits=logits)
         else:
+            eng.decode_model(ses, logits)
             eng.sample_nucleus(ses, ses.out_tokens, ses.top_p, ses.temp, ses.top_k if ses.use_top_k else None,
                                ses.uniforms, keep_mask=keep_mask, logits=logits)
 

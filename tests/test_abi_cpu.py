@@ -22,7 +22,7 @@ def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
     for s in ("mtj_version", "mtj_last_error", "mtj_pack_weight", "mtj_embed", "mtj_layernorm", "mtj_gemm", "mtj_gemv",
               "mtj_attn_prefill", "mtj_attn_decode", "mtj_attn_decode_work_bytes", "mtj_sample_greedy",
-              "mtj_sample_nucleus", "mtj_sample_work_bytes"):
+              "mtj_sample_nucleus", "mtj_sample_work_bytes", "mtj_gemv_greedy"):
         assert s in syms
 
 

@@ -972,6 +972,73 @@ def test_logits_and_cross_entropy_in_one_gemm(L, dt, M, V, K):
                                 a.ptr(ok1), a.ptr(work), nb - 4, S()))
 
 
+@pytest.mark.parametrize("dt,N,K,ln", [("bf16", 50400, 4096, True), ("f32", 1000, 512, False), ("f16", 50400, 1024, True),
+                                       ("bf16", 70, 64, False), ("bf16", 4100, 4096, True)])
+def test_logits_launch_that_is_its_own_greedy_sampler(L, dt, N, K, ln):
+    """mtj_gemv_greedy against mtj_gemv (STORE) followed by mtj_sample_greedy on the same operands: logits, token,
+    token buffer, position and next-step embedding bit for bit, over several launches in a row on one work buffer
+    (every launch leaves it zeroed), with tied maxima (lowest index wins), a maximum in the last row, -0.0 against
+    +0.0 and a NaN among the logits."""
+    a = abi()
+    g = torch.Generator().manual_seed(N + K)
+    code = a.dtype_code(TD[dt])
+    W = (torch.randn(N, K, generator=g) * 0.05).to(TD[dt]).to(DEV)
+    sc, of = (torch.rand(K, generator=g) + 0.5).to(DEV), (torch.randn(K, generator=g) * 0.1).to(DEV)
+    We = (torch.randn(N, 96, generator=g) * 0.02).to(torch.bfloat16).to(DEV)
+    be = torch.randn(96, generator=g).to(DEV)
+    work = torch.zeros(256, dtype=torch.uint8, device=DEV)
+    steps = 6
+    out0 = torch.full((1, steps), -1, dtype=torch.int32, device=DEV)
+    out1 = out0.clone()
+    pos0 = torch.tensor([9], dtype=torch.int32, device=DEV)
+    pos1 = pos0.clone()
+    pos_start = torch.tensor([9], dtype=torch.int32, device=DEV)
+    for t in range(steps):
+        x = torch.randn(K, generator=g).to(DEV)
+        bias = torch.randn(N, generator=g).to(DEV)
+        if t == 1:                                   # two equal maxima far apart, made through the bias of zeroed rows
+            W2 = W.clone(); W2[7] = 0; W2[N - 3] = 0
+            bias[7] = 50.0; bias[N - 3] = 50.0
+        elif t == 2:                                 # the maximum is the very last row
+            W2 = W.clone(); W2[N - 1] = 0
+            bias[N - 1] = 60.0
+        elif t == 3:                                 # all rows zero: +0.0 everywhere but one -0.0; index 0 wins
+            W2 = torch.zeros_like(W)
+            bias.zero_(); bias[0] = -0.0
+        elif t == 4:                                 # a NaN never wins
+            W2 = W.clone(); W2[5] = 0
+            bias[5] = float("nan")
+        else:
+            W2 = W
+        lnp = (a.ptr(sc), a.ptr(of)) if ln else (None, None)
+        lg0, lg1 = torch.empty(1, N, device=DEV), torch.empty(1, N, device=DEV)
+        tok0, tok1 = (torch.zeros(1, dtype=torch.int32, device=DEV) for _ in range(2))
+        xn0, xn1 = torch.zeros(1, 96, device=DEV), torch.zeros(1, 96, device=DEV)
+        ne = a.NextEmbed()
+        ne.w, ne.bias, ne.x_next, ne.d, ne.dtype = a.ptr(We), a.ptr(be), a.ptr(xn0), 96, 1
+        a.check(L.mtj_gemv(a.ptr(x), lnp[0], lnp[1], a.ptr(W2), a.ptr(bias), N, K, code, a.EPI_STORE, a.ptr(lg0), 0, None, None, S()))
+        a.check(L.mtj_sample_greedy(a.ptr(lg0), 1, N, a.ptr(tok0), a.ptr(out0), steps, a.ptr(pos0), a.ptr(pos_start),
+                                    C.byref(ne), S()))
+        ne.x_next = a.ptr(xn1)
+        a.check(L.mtj_gemv_greedy(a.ptr(x), lnp[0], lnp[1], a.ptr(W2), a.ptr(bias), N, K, code, a.ptr(lg1), a.ptr(tok1),
+                                  a.ptr(out1), steps, a.ptr(pos1), a.ptr(pos_start), C.byref(ne), a.ptr(work), S()))
+        torch.cuda.synchronize()
+        assert torch.equal(lg0.view(torch.int32), lg1.view(torch.int32)), t
+        assert tok0.item() == tok1.item(), (t, tok0.item(), tok1.item())
+        assert torch.equal(xn0, xn1) and torch.equal(pos0, pos1), t
+        assert int(work.view(torch.int64).abs().sum()) == 0, t            # ready for the next launch
+        if t == 1:
+            assert tok1.item() == 7
+        if t == 2:
+            assert tok1.item() == N - 1
+        if t == 3:
+            assert tok1.item() == 0
+    assert torch.equal(out0, out1) and (out1 >= 0).all()
+    with pytest.raises(ValueError):
+        a.check(L.mtj_gemv_greedy(a.ptr(x), None, None, a.ptr(W), a.ptr(bias), N, K, code, a.ptr(lg1), a.ptr(tok1), None, 0,
+                                  a.ptr(pos1), a.ptr(pos_start), None, None, S()))
+
+
 def test_greedy_lowest_index_on_ties(L):
     a = abi()
     V = 50400

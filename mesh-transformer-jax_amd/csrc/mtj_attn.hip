@@ -1128,8 +1128,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
       for (int i = 0; i < NI; ++i) {
         int kk = base + (i * 4 + wave) * KPL + sub;
         kk = kk < nk ? kk : nk - 1;
-        kr[buf][i] = *reinterpret_cast<const uint32x4*>(kbase + (int64_t)kk * DH);
-        vr[buf][i] = *reinterpret_cast<const uint32x4*>(vbase + (int64_t)kk * DH);
+        kr[buf][i] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(kbase + (int64_t)kk * DH));
+        vr[buf][i] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(vbase + (int64_t)kk * DH));
       }
     };
     float qv[EPC];

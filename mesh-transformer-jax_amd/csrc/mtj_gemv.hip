@@ -63,8 +63,7 @@ struct gemv_args {
   // ARGMAX only: the greedy sampler behind a STORE of one row of logits
   unsigned long long* am_work;   // [0] best (value image, ~index) so far, [16] arrivals; both 0 between launches
   int32_t* tok;
-  int32_t* out_tokens;
-  int64_t ld_tokens;
+  int32_t* out_tokens;        // row 0 of the token buffer (one sequence)
   int32_t* pos;
   const int32_t* pos_start;
   mtj_next_embed ne;
@@ -751,6 +750,7 @@ extern "C" int mtj_gemv_greedy(const float* x, const float* ln_scale, const floa
                                const float* bias, int64_t N, int64_t K, int dtype, float* logits, int32_t* tok,
                                int32_t* out_tokens, int64_t ld_tokens, int32_t* pos, const int32_t* pos_start,
                                const mtj_next_embed* next, void* work, void* stream) {
+  (void)ld_tokens;
   MTJ_REQUIRE(x && W && logits && tok && pos && pos_start && work, MTJ_EINVAL, "mtj_gemv_greedy: null pointer");
   MTJ_REQUIRE(N > 0 && N < (1ll << 31) && K > 0 && K % 8 == 0, MTJ_EINVAL,
               "mtj_gemv_greedy: K=%lld must be a positive multiple of 8, N below 2^31", (long long)K);
@@ -762,7 +762,7 @@ extern "C" int mtj_gemv_greedy(const float* x, const float* ln_scale, const floa
   a.x = x; a.ln_scale = ln_scale; a.ln_offset = ln_offset; a.W = W; a.bias = bias;
   a.N = N; a.K = K; a.epi = MTJ_EPI_STORE; a.out = logits; a.out_dtype = MTJ_F32;
   a.am_work = reinterpret_cast<unsigned long long*>(work);
-  a.tok = tok; a.out_tokens = out_tokens; a.ld_tokens = ld_tokens; a.pos = pos; a.pos_start = pos_start;
+  a.tok = tok; a.out_tokens = out_tokens; a.pos = pos; a.pos_start = pos_start;   // one row: ld_tokens plays no part
   a.ne = mtj_next_embed{nullptr, nullptr, nullptr, 0, 0};
   if (next && next->w) {
     MTJ_REQUIRE(next->bias && next->x_next && next->d > 0 && (next->dtype == MTJ_F32 || next->dtype == MTJ_BF16), MTJ_EINVAL,

@@ -427,7 +427,9 @@ def nucleaus_filter(logits: np.ndarray, top_p=0.9, top_k=None, acc=np.float64) -
 
     The softmax and its running sum are evaluated in `acc` precision; the contract
     shared with the HIP kernel is acc=float64 (a keep/remove decision then differs from
-    the exact real-number result only if a cumulative mass lies within ~1e-15 of top_p).
+    the exact real-number result only if a cumulative mass lies within ~1e-15 of top_p;
+    the kernel sums the float64 weights exactly as integers of 2^-62, which moves a sum
+    by less than 1.4e-14, so the two agree unless a running sum is that close to its threshold).
     top_p == 1.0 exactly is such a case by construction (the total mass is 1 up to rounding, so
     tail tokens may be removed depending on summation order); "keep everything" is top_p > 1.
     Returns the filtered float32 logits in token order."""

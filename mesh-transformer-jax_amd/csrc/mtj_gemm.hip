@@ -652,11 +652,19 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const gemm_args a) {
   // my K range (split-K: blockIdx.y; the whole of K otherwise), in k-tiles
   const int kt0 = (int)((int64_t)blockIdx.y * (a.K / BK) / a.splits);
   const int KT = (int)((int64_t)(blockIdx.y + 1) * (a.K / BK) / a.splits) - kt0;
+  // Every operand row of a k-tile lies at the same offset inside its row, and the rows are a power of two apart: when
+  // the whole chip walks k in step it asks at any moment for addresses that fall into few memory channels.  With one
+  // group of row tiles (a short prompt: every XCD then has its own range of column tiles, and all workgroups run at
+  // once) the walk starts an eighth of the k range further on in every eighth of the column tiles and wraps around:
+  // the workgroups of an XCD still walk together and share their activation panels through its L2, the XCDs do not.
+  // The start depends on the column tile alone.
+  const int krot = tiles_m <= 8 ? (int)((((int64_t)tn * 8) / tiles_n) * KT / 8) : 0;
 
   // set 0: A first half, 1: W first half, 2: W second half, 3: A second half
   auto issue = [&](int st, int kt, auto SET_) {
     constexpr int set = decltype(SET_)::value;
-    const int koff = (kt0 + kt) * ROWB;
+    const int kr = kt + krot;
+    const int koff = (kt0 + (kr >= KT ? kr - KT : kr)) * ROWB;
     // a k-tile beyond the range is requested all the same (the wait counts stay the same in every k-tile) but with an
     // offset far outside the buffer: such a load fetches nothing and writes zeros into a stage that is not read again
     const int beyond = kt < KT ? 0 : 0x40000000;

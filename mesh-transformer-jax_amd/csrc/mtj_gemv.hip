@@ -494,6 +494,7 @@ __global__ __launch_bounds__(1024) void gemv_outatt_kernel(const outatt_args oa)
     for (int i = 0; i < NI; ++i) {
       int kk = kb + (i * 16 + wave) * KPL + sub;
       kk = kk < nk ? kk : nk - 1;
+      // streaming loads, like the weights: nothing of the window is read twice in a step
       kr[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(kbase + (int64_t)kk * DH));
       vr[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32x4*>(vbase + (int64_t)kk * DH));
     }
